@@ -1,0 +1,133 @@
+/*
+ * intfa.h - C ABI of the MI355X (gfx950) INT8 FlashAttention forward library (libintfa.so).
+ *
+ * The reference ships no host API for this path: its Python entry points launch Triton kernels
+ * directly (flash_atten_full_int8.py:186-221, flash_atten_int8.py:181-215, flash_atten_fp.py:155-187)
+ * and its CUDA sources stop at the templates
+ *     run_mha_fwd_full_qi8_<T,128>(Flash_fwd_params&, cudaStream_t)      (csrc/flash.h:205-208)
+ * which take one parameter block plus a stream.  The entry points below keep that shape - one plain-C
+ * parameter block (the counterpart of Qkv_params / Flash_fwd_params, csrc/flash.h:24-159) and a stream -
+ * with the tensor conventions of the Python entry points ([Z,H,N,d] tensors, [Z,H,N] per-token scales,
+ * [Z,H] value scale).
+ *
+ * Conventions of every entry point:
+ *   - all pointers are DEVICE pointers borrowed for the duration of the enqueued work;
+ *   - strides are in ELEMENTS of the tensor they describe; the head dimension is contiguous (stride 1);
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the null stream); the call does not
+ *     synchronise, allocate or free;
+ *   - return value: 0 on success, a negative INTFA_ERR_* for a rejected argument, a positive hipError_t when
+ *     the launch itself failed;
+ *   - re-entrant and thread-safe for distinct streams (no mutable global state).
+ */
+#ifndef INTFA_H_
+#define INTFA_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define INTFA_VERSION 1
+
+/* element types of scales / float tensors */
+enum { INTFA_F16 = 0, INTFA_BF16 = 1, INTFA_F32 = 2 };
+
+/* rounding used when P is requantised to int8 (full-int8 path) */
+enum {
+    /* 127*p evaluated in fp32 and rounded to nearest-even by one hardware convert */
+    INTFA_PROUND_RNE = 0,
+    /* the reference's fp16 sequence: fp16(p) * 127, + 0.5, truncating cast (flash_atten_full_int8.py:49-51) */
+    INTFA_PROUND_REFERENCE = 1
+};
+
+enum {
+    INTFA_OK = 0,
+    INTFA_ERR_NULL = -1,          /* a required pointer is NULL */
+    INTFA_ERR_HEAD_DIM = -2,      /* head_dim not supported by the kernels */
+    INTFA_ERR_SEQLEN = -3,        /* seqlen not a positive multiple of the key block (128) */
+    INTFA_ERR_ALIGN = -4,         /* pointer or row stride not 16-byte aligned */
+    INTFA_ERR_DTYPE = -5,         /* unknown dtype enum */
+    INTFA_ERR_WORKSPACE = -6,     /* workspace missing or too small for the requested split count */
+    INTFA_ERR_SHAPE = -7,         /* batch/heads not positive, or sizes overflow 32-bit block indices */
+    INTFA_ERR_SPLITS = -8         /* num_splits out of range */
+};
+
+/*
+ * Parameter block shared by the three forward variants.  Unused members of a variant are ignored
+ * (q_scale/k_scale for the fp16 variant, v_scale for the half-int8 and fp16 variants).
+ *
+ *   variant      q, k            v               out
+ *   full-int8    int8            int8            out_dtype (fp16 as in the reference, or bf16)
+ *   half-int8    int8            fp16 or bf16    out_dtype (= v's type)
+ *   fp16         fp16 or bf16    same as q       same as q
+ */
+typedef struct intfa_fwd_params {
+    const void* q;            /* [batch, heads, seqlen, head_dim] */
+    const void* k;
+    const void* v;
+    void*       out;
+    const void* q_scale;      /* [batch, heads, seqlen], scale_dtype */
+    const void* k_scale;      /* [batch, heads, seqlen], scale_dtype */
+    const void* v_scale;      /* [batch, heads], scale_dtype */
+    float*      lse;          /* optional [batch, heads, seqlen] contiguous: m + log2(l), base-2 as the
+                                 reference's M (flash_atten_int8.py:172-175); NULL = not written */
+
+    int64_t q_stride_b, q_stride_h, q_stride_n;
+    int64_t k_stride_b, k_stride_h, k_stride_n;
+    int64_t v_stride_b, v_stride_h, v_stride_n;
+    int64_t o_stride_b, o_stride_h, o_stride_n;
+    int64_t qs_stride_b, qs_stride_h, qs_stride_n;
+    int64_t ks_stride_b, ks_stride_h, ks_stride_n;
+    int64_t vs_stride_b, vs_stride_h;
+
+    int32_t batch, heads, seqlen, head_dim;
+    int32_t scale_dtype;      /* INTFA_F16 / INTFA_BF16 / INTFA_F32 */
+    int32_t io_dtype;         /* type of out (and of fp q/k/v): INTFA_F16 or INTFA_BF16 */
+    int32_t causal;           /* 0 / 1; queries and keys share positions (seqlen_q == seqlen_k) */
+    float   sm_scale;
+    int32_t p_round;          /* INTFA_PROUND_* (full-int8 only) */
+
+    int32_t num_splits;       /* <= 1: single pass; > 1: split-KV partials + combine (needs workspace) */
+    void*   workspace;        /* device scratch of at least intfa_fwd_workspace_bytes() bytes, or NULL */
+    size_t  workspace_bytes;
+} intfa_fwd_params;
+
+/* Library/ABI version (INTFA_VERSION of the build). */
+int intfa_version(void);
+
+/* Human-readable text for a negative return code; for a positive one returns "hip error". */
+const char* intfa_error_string(int code);
+
+/* Key-block length the kernels quantise P against (the reference's BLOCK_N, an autotuned value there:
+ * configs.py:13-19).  A bit-faithful CPU evaluation must use the same value. */
+int intfa_block_n(void);
+
+/* Bytes of workspace the forward needs for p->num_splits (0 when num_splits <= 1). */
+size_t intfa_fwd_workspace_bytes(const intfa_fwd_params* p);
+
+/* attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal, sm_scale) -> o
+ * replaces _attention_full_int8.forward + _attn_fwd_full_int8 (flash_atten_full_int8.py:73-221);
+ * native counterpart run_mha_fwd_full_qi8_ (csrc/flash_fwd_launch_template.h:503-523). */
+int intfa_fwd_full_int8(const intfa_fwd_params* p, void* stream);
+
+/* attention_int8(q, k, v, q_scale, k_scale, causal, sm_scale) -> o
+ * replaces _attention_int8.forward + _attn_fwd_int8 (flash_atten_int8.py:68-215);
+ * native counterpart run_mha_fwd_half_qi8_ (csrc/flash_fwd_launch_template.h:469-501). */
+int intfa_fwd_half_int8(const intfa_fwd_params* p, void* stream);
+
+/* attention(q, k, v, causal, sm_scale) -> o
+ * replaces _attention.forward + _attn_fwd (flash_atten_fp.py:62-187);
+ * native counterpart run_mha_fwd_<T,128> (csrc/flash.h:205). */
+int intfa_fwd_fp16(const intfa_fwd_params* p, void* stream);
+
+/* Debug export of the int32 accumulators S = Q8 K8^T produced by the same MFMA tile code the forward
+ * uses (flash_atten_full_int8.py:36).  s_out is [batch, heads, seqlen, seqlen] int32, contiguous.
+ * Uses q, k and their strides, batch, heads, seqlen, head_dim of the block. */
+int intfa_debug_qk_int32(const intfa_fwd_params* p, int32_t* s_out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INTFA_H_ */

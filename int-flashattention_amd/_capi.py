@@ -1,0 +1,74 @@
+"""ctypes binding of libintfa.so (the C ABI declared in include/intfa.h).
+
+The library is built in-tree by ``build.py`` (hipcc, gfx950).  There is no fallback: when the shared
+object is absent or does not load, every entry point raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libintfa.so")
+
+INTFA_F16, INTFA_BF16, INTFA_F32 = 0, 1, 2
+PROUND_RNE, PROUND_REFERENCE = 0, 1
+
+
+class FwdParams(ctypes.Structure):
+    """Mirror of ``intfa_fwd_params`` (include/intfa.h); field order and types must match exactly."""
+    _fields_ = (
+        [(n, ctypes.c_void_p) for n in ("q", "k", "v", "out", "q_scale", "k_scale", "v_scale", "lse")]
+        + [(n, ctypes.c_int64) for n in (
+            "q_stride_b", "q_stride_h", "q_stride_n",
+            "k_stride_b", "k_stride_h", "k_stride_n",
+            "v_stride_b", "v_stride_h", "v_stride_n",
+            "o_stride_b", "o_stride_h", "o_stride_n",
+            "qs_stride_b", "qs_stride_h", "qs_stride_n",
+            "ks_stride_b", "ks_stride_h", "ks_stride_n",
+            "vs_stride_b", "vs_stride_h")]
+        + [(n, ctypes.c_int32) for n in ("batch", "heads", "seqlen", "head_dim", "scale_dtype", "io_dtype", "causal")]
+        + [("sm_scale", ctypes.c_float), ("p_round", ctypes.c_int32), ("num_splits", ctypes.c_int32),
+           ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t)]
+    )
+
+
+EXPORTS = ("intfa_version", "intfa_error_string", "intfa_block_n", "intfa_fwd_workspace_bytes",
+           "intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16", "intfa_debug_qk_int32")
+
+_lib = None
+
+
+def load():
+    """Loads libintfa.so once and declares the prototypes.  Raises if the library is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} not found: the HIP extension is not built. Run `python -m int_flashattention_amd.build` "
+            "(needs hipcc). There is no CPU or PyTorch fallback for the attention kernels.")
+    lib = ctypes.CDLL(LIB_PATH)
+    pp = ctypes.POINTER(FwdParams)
+    lib.intfa_version.restype = ctypes.c_int
+    lib.intfa_version.argtypes = []
+    lib.intfa_block_n.restype = ctypes.c_int
+    lib.intfa_block_n.argtypes = []
+    lib.intfa_error_string.restype = ctypes.c_char_p
+    lib.intfa_error_string.argtypes = [ctypes.c_int]
+    lib.intfa_fwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.intfa_fwd_workspace_bytes.argtypes = [pp]
+    for name in ("intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16"):
+        fn = getattr(lib, name)
+        fn.restype = ctypes.c_int
+        fn.argtypes = [pp, ctypes.c_void_p]
+    lib.intfa_debug_qk_int32.restype = ctypes.c_int
+    lib.intfa_debug_qk_int32.argtypes = [pp, ctypes.c_void_p, ctypes.c_void_p]
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().intfa_error_string(rc).decode()
+        raise RuntimeError(f"{what} failed with code {rc}: {msg}")

@@ -1,0 +1,126 @@
+// Device-side building blocks shared by the forward kernels (gfx950 / CDNA4 only).
+//
+// Tile geometry used throughout:
+//   * a workgroup is 4 wavefronts (256 threads) and owns BLOCK_M = 128 query rows, 32 per wavefront;
+//   * keys are consumed in blocks of BLOCK_N = 128, each handled as 4 sub-tiles of 32 keys;
+//   * the score tile is computed TRANSPOSED, S^T = K Q^T, with v_mfma_i32_32x32x32_i8: a lane then holds one
+//     query column (lane % 32) and 16 keys, so row max / row sum are in-lane reductions plus one exchange
+//     between lane l and lane l^32, and the accumulator registers run along the key axis - the contraction
+//     axis of P V - which lets P be packed to int8 in-lane and fed straight back as an MFMA B operand.
+//
+// MFMA register layouts relied on (verified on hardware against a CPU matmul):
+//   v_mfma_i32_32x32x32_i8   A: lane (m = l%32, h = l/32) holds bytes k = 16h .. 16h+15 of row m
+//                            B: lane (n = l%32, h)        holds bytes k = 16h .. 16h+15 of column n
+//                            D: lane (n = l%32, h) register r holds row m = 8*(r/4) + 4*h + r%4
+//   v_mfma_f32_32x32x16_f16  same with 8 halves per lane, k = 8h .. 8h+7
+//   ds_read_b64_tr_b8        inside each group of 16 lanes, result lane i byte j = byte (i%8) of the 8 bytes
+//                            addressed by lane (2j + i/8) of the group
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace intfa {
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+
+#define INTFA_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+#define INTFA_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
+
+constexpr int kBlockM = 128;
+constexpr int kBlockN = 128;
+constexpr int kThreads = 256;
+constexpr float kLog2_127 = 6.98868468677f;   // log2(127)
+
+// Kernel-side parameter block (byte strides, resolved pointers).
+struct KParams {
+    const char* q; const char* k; const char* v; char* out;
+    const char* q_scale; const char* k_scale; const char* v_scale;
+    float* lse;
+    int32_t* s_dump;                       // debug: int32 S [B,H,N,N]
+    float* o_part; float* lse_part;        // split-KV partials [S,B,H,N,D] fp32 / [S,B,H,N]
+    int64_t q_sb, q_sh, q_sn;              // bytes
+    int64_t k_sb, k_sh, k_sn;
+    int64_t v_sb, v_sh, v_sn;
+    int64_t o_sb, o_sh, o_sn;
+    int64_t qs_sb, qs_sh, qs_sn;           // elements
+    int64_t ks_sb, ks_sh, ks_sn;
+    int64_t vs_sb, vs_sh;
+    int32_t batch, heads, seqlen, head_dim;
+    int32_t scale_dtype, causal, num_splits, blocks_per_split;
+    float qk_scale_log2;                   // sm_scale * log2(e)
+};
+
+__device__ __forceinline__ float load_scale(const char* base, int64_t idx, int dtype) {
+    if (dtype == 0) return (float)((const _Float16*)base)[idx];
+    if (dtype == 1) return __builtin_bit_cast(float, ((uint32_t)((const uint16_t*)base)[idx]) << 16);
+    return ((const float*)base)[idx];
+}
+
+// ---- LDS swizzles.  A tile row is D bytes; its 16-byte chunks are XOR-permuted with a function of the row so
+// that the 8 rows touched together by one group of lanes fall into 8 different bank groups.
+// K rows are read by 8 consecutive lanes as 8 consecutive rows.
+template <int ROW_BYTES> __device__ __forceinline__ int swz_k(int row) {
+    if (ROW_BYTES >= 128) return row & 7;
+    return (row >> 1) & 3;                       // 64-byte rows: two rows share a 128-byte line
+}
+// V rows are read by the transposing load as rows {0,1,2,3,8,9,10,11} + 4h of a 32-key sub-tile.
+template <int ROW_BYTES> __device__ __forceinline__ int swz_v(int row) {
+    if (ROW_BYTES >= 128) return (row & 3) | ((row >> 1) & 4);
+    return ((row >> 1) & 1) | ((row >> 2) & 2);
+}
+
+// Asynchronous copy of one 128-row tile (ROW_BYTES bytes per row) from global memory straight into LDS with
+// global_load_lds_dwordx4: every wave instruction moves 64 x 16 bytes into 1 KiB of consecutive LDS, so the
+// swizzle is applied on the GLOBAL side (which chunk a lane fetches).  The four waves split the instructions.
+// Addressing is split into a wave-uniform 64-bit base (SGPRs) and a per-lane 32-bit offset.  The swizzle of a
+// row depends on the row's low four bits only; wave w issues instructions w, w+4, w+8, ... whose first rows
+// differ by multiples of 4*RPI rows, so a lane needs one offset when 4*RPI >= 16 and two otherwise.
+template <int ROW_BYTES, bool IS_V> struct TileLoadLane {
+    static constexpr int CH = ROW_BYTES / 16;        // 16-byte chunks per row
+    static constexpr int RPI = 64 / CH;              // rows per wave instruction
+    static constexpr int NINST = kBlockN * CH / 64;  // wave instructions per tile
+    static constexpr int NV = (4 * RPI >= 16) ? 1 : 16 / (4 * RPI);
+    static_assert(RPI >= 2 && RPI <= 16 && NINST % 4 == 0, "unsupported row size");
+    uint32_t off[NV];
+};
+template <int ROW_BYTES, bool IS_V>
+__device__ __forceinline__ TileLoadLane<ROW_BYTES, IS_V> tile_load_lane(uint32_t row_stride, int wave, int lane) {
+    using T = TileLoadLane<ROW_BYTES, IS_V>;
+    constexpr int SM = (T::CH < 8 ? T::CH : 8) - 1;
+    const int rsub = lane / T::CH, cp = lane % T::CH;
+    T t;
+#pragma unroll
+    for (int v = 0; v < T::NV; ++v) {
+        const int row = (v * 4 + wave) * T::RPI + rsub;
+        const int f = (IS_V ? swz_v<ROW_BYTES>(row) : swz_k<ROW_BYTES>(row)) & SM;
+        t.off[v] = (uint32_t)rsub * row_stride + (uint32_t)((cp ^ f) << 4);
+    }
+    return t;
+}
+template <int ROW_BYTES, bool IS_V>
+__device__ __forceinline__ void issue_tile_load(const char* gtile, uint32_t row_stride, char* lds_tile, int wave,
+                                                const TileLoadLane<ROW_BYTES, IS_V>& ln) {
+    using T = TileLoadLane<ROW_BYTES, IS_V>;
+#pragma unroll
+    for (int it = 0; it < T::NINST / 4; ++it) {
+        const int i = it * 4 + wave;                 // wave-uniform instruction index
+        const char* g = gtile + (uint64_t)(i * T::RPI) * row_stride;
+        __builtin_amdgcn_global_load_lds(INTFA_GLB(g + ln.off[it % T::NV]), INTFA_LDS(lds_tile + i * 1024), 16, 0, 0);
+    }
+}
+
+__device__ __forceinline__ float wave_half_swap(float x) {      // value held by lane l ^ 32
+    return __shfl_xor(x, 32);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+}  // namespace intfa

@@ -1,0 +1,23 @@
+"""Drop-in for the reference module of the same name: ``attention_full_int8`` (flash_atten_full_int8.py:186-223)."""
+import torch
+
+from . import _capi
+from ._host import launch_forward
+
+
+def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, *, out_dtype=torch.float16,
+                        num_splits=1, p_round="rne", return_lse=False):
+    """Full-int8 attention forward.
+
+    q, k, v: int8 [Z, H, N, d]; q_scale, k_scale: [Z, H, N] per-token scales; v_scale: [Z, H];
+    returns a new contiguous [Z, H, N, d] tensor, fp16 as in the reference (flash_atten_full_int8.py:194-195)
+    unless ``out_dtype=torch.bfloat16`` is asked for.  Causal runs use the correct running-max hand-off between
+    the off-diagonal and diagonal stages (as flash_atten_int8.py:157-166 does), not the reference's
+    full-int8 behaviour, which restarts from -inf (flash_atten_full_int8.py:166,175).
+
+    ``p_round``: "rne" folds 127 into the exponent and rounds to nearest-even; "reference" reproduces the
+    fp16 sequence of flash_atten_full_int8.py:49-51.
+    """
+    pr = {"rne": _capi.PROUND_RNE, "reference": _capi.PROUND_REFERENCE}[p_round]
+    return launch_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, out_dtype,
+                          num_splits=num_splits, p_round=pr, return_lse=return_lse)

@@ -1,0 +1,300 @@
+"""CPU oracle for the INT8 FlashAttention forward path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, in plain PyTorch on the CPU, the arithmetic that the reference's three
+forward entry points perform.  It is the checker for the HIP kernels: only ``tests/``,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import it.  The product
+package never does, and it fails loudly when its HIP library is missing.
+
+What each function follows in the reference (paths relative to the reference checkout):
+
+* ``quant_pertoken``           - benchmark.py:96-100
+* ``quant_pertensor``          - benchmark.py:102-107
+* ``mean_relative_error``      - benchmark.py:110-122 (``calc_num=4`` reproduces it; ``None`` = all elements)
+* ``attention_exact``          - benchmark.py:152-154 (non-causal) and benchmark.py:224-230 (causal tril mask)
+* ``qk_int32``                 - flash_atten_full_int8.py:36 (the int32 accumulator of ``tl.dot(q, k)``)
+* ``attention_full_int8``      - flash_atten_full_int8.py:9-71 (tile loop), :148-182 (init + epilogue); the causal
+                                 hand-off of the running max follows flash_atten_int8.py:66,157,166 because the
+                                 full-int8 file drops it (flash_atten_full_int8.py:71,166,175 return only acc, l_i)
+* ``attention_int8``           - flash_atten_int8.py:9-66, :140-176 (also returns M = m + log2(l), :172-175)
+* ``attention_fp``             - flash_atten_fp.py:9-60, :115-150
+* ``splitkv_ranges``           - csrc/flash_fwd_kernel.h:503-511 (key-block range of a split)
+* ``splitkv_combine``          - csrc/flash_fwd_kernel.h:1212-1235 (log-sum-exp over splits), :1264-1283 (weighted sum)
+
+Free parameters of the reference that are fixed here by argument: ``block_m``/``block_n`` (the reference
+autotunes them, and its result depends on ``block_n`` because P is quantised against the running
+maximum of the blocks seen so far) and the key-block order (ascending, as in the Triton loop).
+
+How every function is pinned (tests/test_oracle.py):
+
+* quantisers: closed form (absmax/127, round-half-even), invariants (every row reaches +-127), brute force.
+* ``qk_int32``: exact integer matmul compared with a pure-Python triple loop and with numpy int64.
+* P requantisation ``p_requant_reference``: exhaustive over all fp16 values in [0, 1] against a scalar
+  restatement using ``numpy.float16`` arithmetic.
+* online softmax: ``block_n = N`` must reproduce ``torch.softmax``; any ``block_n`` gives the same (m, l) up to
+  fp32 rounding; with every scale equal to one the path is plain integer attention; with V constant the output
+  is that constant times sum(P8)/(127 l).
+* causal: equality with a dense tril-masked evaluation; first row attends to key 0 only.
+* split-KV: any split count agrees with one split to fp32 rounding.
+
+The reference holds no golden vectors for this path (its only test asserts the fp16 forward with
+atol=1e-2, benchmark.py:242), so none are used.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+LOG2E = 1.44269504  # the literal used at flash_atten_full_int8.py:157
+
+
+# --------------------------------------------------------------------------------------------------
+# quantisers and error measures (benchmark.py)
+# --------------------------------------------------------------------------------------------------
+def quant_pertoken(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """benchmark.py:96-100: per-row symmetric int8, scale = absmax/127 in the input dtype."""
+    x_max, _ = torch.abs(x).max(dim=-1)
+    x_scale = x_max / 127
+    ret = torch.round(x / x_scale[:, :, :, None]).to(torch.int8)
+    return ret, x_scale
+
+
+def quant_pertensor(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """benchmark.py:102-107: one scale per (batch, head) slice."""
+    x_max, _ = torch.abs(x).max(dim=-1)
+    x_max, _ = torch.max(x_max, dim=-1)
+    x_scale = x_max / 127
+    ret = torch.round(x / x_scale[:, :, None, None]).to(torch.int8)
+    return ret, x_scale
+
+
+def mean_relative_error(a: torch.Tensor, b: torch.Tensor, calc_num: Optional[int] = None) -> float:
+    """benchmark.py:110-122: mean(|b - a| / (|b| + 1e-5)); the reference looks at the last 4 elements only."""
+    assert a.shape == b.shape
+    m1 = b.reshape(-1).float()
+    m2 = a.reshape(-1).float()
+    if calc_num is not None:
+        m1, m2 = m1[-calc_num:], m2[-calc_num:]
+    return (torch.abs(m1 - m2) / (torch.abs(m1) + 1e-5)).mean().item()
+
+
+def attention_exact(q, k, v, causal: bool, sm_scale: float) -> torch.Tensor:
+    """benchmark.py:152-154 / :224-230: softmax(QK^T * sm_scale) V with an fp32 softmax.
+
+    Computed in fp32 throughout on the CPU (the reference does the two matmuls in fp16 on the GPU);
+    P is rounded to the input dtype before the second matmul as the reference does.
+    """
+    qf, kf, vf = q.float(), k.float(), v.float()
+    p = torch.matmul(qf, kf.transpose(2, 3)) * sm_scale
+    if causal:
+        n = q.shape[2]
+        mask = torch.tril(torch.ones((n, n), dtype=torch.bool))
+        p = p.masked_fill(~mask, float("-inf"))
+    p = torch.softmax(p, dim=-1).to(q.dtype if q.dtype.is_floating_point else torch.float16).float()
+    return torch.matmul(p, vf).to(q.dtype if q.dtype.is_floating_point else torch.float16)
+
+
+# --------------------------------------------------------------------------------------------------
+# integer pieces
+# --------------------------------------------------------------------------------------------------
+def _int_matmul(a8: torch.Tensor, b8: torch.Tensor) -> torch.Tensor:
+    """Exact integer matmul a8 @ b8 returned as fp32 holding integers.
+
+    fp32 GEMM is exact here: every partial sum is an integer below 2**24 (|a|,|b| <= 128, inner
+    dimension <= 1024), so no rounding occurs in any summation order.
+    """
+    assert a8.shape[-1] <= 1024
+    return torch.matmul(a8.float(), b8.float())
+
+
+def qk_int32(q8: torch.Tensor, k8: torch.Tensor) -> torch.Tensor:
+    """flash_atten_full_int8.py:36: S = Q8 K8^T accumulated in int32, shape [B,H,N,N]."""
+    return _int_matmul(q8, k8.transpose(2, 3)).to(torch.int32)
+
+
+def p_requant_reference(p: torch.Tensor) -> torch.Tensor:
+    """flash_atten_full_int8.py:49-51: p.to(fp16); p * 127; (p + 0.5).to(int8) - all in fp16, truncating cast.
+
+    Returns fp32 holding the integers 0..127.
+    """
+    p16 = p.to(torch.float16)
+    p16 = p16 * 127          # fp16 product, rounded to fp16
+    p16 = p16 + 0.5          # fp16 sum, rounded to fp16
+    return torch.trunc(p16.float())
+
+
+def p_requant_rne(p: torch.Tensor) -> torch.Tensor:
+    """Round-to-nearest-even of 127 p in fp32: what one hardware float->u8 convert of 127 p yields.
+
+    Not the reference's formula; kept so tests can measure how far the two roundings are apart.
+    """
+    return torch.clamp(torch.round(p * 127.0), 0, 255)
+
+
+# --------------------------------------------------------------------------------------------------
+# the blocked forward (all three variants share the loop skeleton)
+# --------------------------------------------------------------------------------------------------
+def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float,
+                     block_m: int, block_n: int, key_lo: int = 0, key_hi: Optional[int] = None,
+                     p_requant=p_requant_reference, pv_dtype=torch.float16):
+    """Runs the reference's tile loop over key blocks [key_lo, key_hi) for every query row at once.
+
+    Rows are grouped in tiles of ``block_m`` as the reference's programs are; for a causal run a tile sees
+    the key blocks below its first row without a mask (stage 1) and the blocks of its own row range with the
+    mask (stage 2), flash_atten_full_int8.py:18-25.  Returns fp32 (acc, l, m) with acc un-normalised.
+    """
+    B, H, N, D = q.shape
+    key_hi = N if key_hi is None else key_hi
+    assert N % block_m == 0 and N % block_n == 0 and block_m % block_n == 0
+    assert key_lo % block_n == 0 and key_hi % block_n == 0
+    qk_scale = float(torch.tensor(sm_scale, dtype=torch.float32) * torch.tensor(LOG2E, dtype=torch.float32))
+    m = torch.full((B, H, N), float("-inf"), dtype=torch.float32)
+    l = torch.ones((B, H, N), dtype=torch.float32)          # flash_atten_full_int8.py:153
+    acc = torch.zeros((B, H, N, D), dtype=torch.float32)
+    int_qk = variant in ("full", "half")
+    if int_qk:
+        qs = q_scale.float()
+        ks = k_scale.float()
+    if variant == "full":
+        vs = v_scale.float()[:, :, None, None]
+    rows = torch.arange(N)
+
+    for start_n in range(key_lo, key_hi, block_n):
+        kj = k[:, :, start_n:start_n + block_n]
+        vj = v[:, :, start_n:start_n + block_n]
+        if causal:
+            tile = start_n // block_m
+            segments = [(tile * block_m, (tile + 1) * block_m, True), ((tile + 1) * block_m, N, False)]
+        else:
+            segments = [(0, N, False)]
+        for r0, r1, masked in segments:
+            if r0 >= r1:
+                continue
+            qi = q[:, :, r0:r1]
+            if int_qk:
+                qk = _int_matmul(qi, kj.transpose(2, 3))                     # int32 accumulator, :36
+                qk = qk * qs[:, :, r0:r1, None]                              # :37
+                qk = qk * ks[:, :, None, start_n:start_n + block_n]          # :38
+            else:
+                qk = torch.matmul(qi.float(), kj.float().transpose(2, 3))    # flash_atten_fp.py:33
+            m_i = m[:, :, r0:r1]
+            if masked:                                                       # :39-43
+                keep = rows[r0:r1, None] >= (start_n + torch.arange(block_n))[None, :]
+                qk = qk * qk_scale + torch.where(keep, 0.0, -1.0e6)
+                m_ij = torch.maximum(m_i, qk.max(dim=-1).values)
+                qk = qk - m_ij[..., None]
+            else:                                                            # :44-46
+                m_ij = torch.maximum(m_i, qk.max(dim=-1).values * qk_scale)
+                qk = qk * qk_scale - m_ij[..., None]
+            p = torch.exp2(qk)                                               # :47
+            l_ij = p.sum(dim=-1)                                             # :48
+            alpha = torch.exp2(m_i - m_ij)                                   # :53
+            l[:, :, r0:r1] = l[:, :, r0:r1] * alpha + l_ij                   # :54
+            a = acc[:, :, r0:r1] * alpha[..., None]                          # :56
+            if variant == "full":
+                p8 = p_requant(p)                                            # :49-51
+                tmp = _int_matmul(p8, vj)                                    # :59 int32 accumulator
+                tmp = tmp * vs / 127                                         # :61
+                a = a + tmp                                                  # :62
+            else:
+                pl = p.to(pv_dtype).float()                                  # flash_atten_int8.py:58
+                a = a + torch.matmul(pl, vj.float())                         # :59 fp32 accumulate
+            acc[:, :, r0:r1] = a
+            m[:, :, r0:r1] = m_ij                                            # :67
+    return acc, l, m
+
+
+def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float, *,
+                        block_m: int = 128, block_n: int = 128, out_dtype=torch.float16,
+                        p_requant=p_requant_reference, return_lse: bool = False):
+    """Full-int8 forward, flash_atten_full_int8.py (see module docstring for line map)."""
+    acc, l, m = _blocked_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale,
+                                 block_m, block_n, p_requant=p_requant)
+    o = (acc / l[..., None]).to(out_dtype)                                   # :181-182
+    if return_lse:
+        return o, m + torch.log2(l)
+    return o
+
+
+def attention_int8(q, k, v, q_scale, k_scale, causal: bool, sm_scale: float, *,
+                   block_m: int = 128, block_n: int = 128, out_dtype=torch.float16, return_lse: bool = False):
+    """Half-int8 forward, flash_atten_int8.py: int8 QK^T, P cast to V's dtype, fp32-accumulated PV."""
+    acc, l, m = _blocked_forward("half", q, k, v, q_scale, k_scale, None, causal, sm_scale,
+                                 block_m, block_n, pv_dtype=v.dtype)
+    o = (acc / l[..., None]).to(out_dtype)
+    if return_lse:
+        return o, m + torch.log2(l)                                          # :172-175
+    return o
+
+
+def attention_fp(q, k, v, causal: bool, sm_scale: float, *, block_m: int = 128, block_n: int = 128,
+                 return_lse: bool = False):
+    """fp16/bf16 forward, flash_atten_fp.py; output has q's dtype (:162)."""
+    acc, l, m = _blocked_forward("fp", q, k, v, None, None, None, causal, sm_scale,
+                                 block_m, block_n, pv_dtype=q.dtype)
+    o = (acc / l[..., None]).to(q.dtype)
+    if return_lse:
+        return o, m + torch.log2(l)
+    return o
+
+
+# --------------------------------------------------------------------------------------------------
+# split-KV (the reference has it for fp16 only; csrc/kernel_traits.h:199 leaves the int8 version open)
+# --------------------------------------------------------------------------------------------------
+def splitkv_ranges(n_keys: int, block_n: int, num_splits: int):
+    """csrc/flash_fwd_kernel.h:503-511: key-block range [min, max) of each split."""
+    n_blocks = (n_keys + block_n - 1) // block_n
+    per = (n_blocks + num_splits - 1) // num_splits
+    return [(s * per, min(n_blocks, (s + 1) * per)) for s in range(num_splits)]
+
+
+def splitkv_combine(o_parts: torch.Tensor, lse_parts: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """csrc/flash_fwd_kernel.h:1212-1235, :1264-1283 in base 2 (the kernels keep log2-domain statistics).
+
+    o_parts [S,B,H,N,D] fp32 are partial outputs already divided by their own l; lse_parts [S,B,H,N]
+    are m + log2(l), -inf for a split that saw no key.
+    """
+    lse_max = lse_parts.max(dim=0).values
+    lse_max = torch.where(torch.isinf(lse_max), torch.zeros_like(lse_max), lse_max)
+    lse_sum = torch.exp2(lse_parts - lse_max).sum(dim=0)
+    lse = torch.where(lse_sum == 0, torch.full_like(lse_sum, float("inf")), torch.log2(lse_sum) + lse_max)
+    w = torch.exp2(lse_parts - lse)
+    return (w[..., None] * o_parts).sum(dim=0), lse
+
+
+def attention_full_int8_splitkv(q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float, num_splits: int, *,
+                                block_m: int = 128, block_n: int = 128, out_dtype=torch.float16):
+    """Full-int8 forward evaluated as ``num_splits`` independent key ranges merged by ``splitkv_combine``."""
+    B, H, N, D = q.shape
+    o_parts, lse_parts = [], []
+    for b0, b1 in splitkv_ranges(N, block_n, num_splits):
+        if b0 >= b1:
+            o_parts.append(torch.zeros((B, H, N, D)))
+            lse_parts.append(torch.full((B, H, N), float("-inf")))
+            continue
+        acc, l, m = _blocked_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale,
+                                     block_m, block_n, key_lo=b0 * block_n, key_hi=b1 * block_n)
+        seen = ~torch.isinf(m)                       # causal rows above the split's range saw no key
+        o_parts.append(torch.where(seen[..., None], acc / l[..., None], torch.zeros_like(acc)))
+        lse_parts.append(torch.where(seen, m + torch.log2(l), torch.full_like(m, float("-inf"))))
+    o, _ = splitkv_combine(torch.stack(o_parts), torch.stack(lse_parts))
+    return o.to(out_dtype)
+
+
+# --------------------------------------------------------------------------------------------------
+# synthetic inputs of the benchmark configurations
+# --------------------------------------------------------------------------------------------------
+def make_inputs(B: int, H: int, N: int, D: int, *, seed: int = 20, dtype=torch.float16, std: float = 1.0,
+                k_outlier_frac: float = 0.0, k_outlier_gain: float = 20.0):
+    """Seeded N(0, std) Q, K, V in ``dtype``; optionally a fraction of K's channels is multiplied by a gain."""
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn((B, H, N, D), generator=g) * std).to(dtype)
+    k = torch.randn((B, H, N, D), generator=g) * std
+    v = (torch.randn((B, H, N, D), generator=g) * std).to(dtype)
+    cols = []
+    if k_outlier_frac > 0:
+        n_out = max(1, int(round(D * k_outlier_frac)))
+        cols = torch.randperm(D, generator=g)[:n_out].tolist()
+        k[..., cols] *= k_outlier_gain
+    return q, k.to(dtype), v, cols
