@@ -1,0 +1,120 @@
+"""CPU-side checks of the drop-in boundary: the C ABI library loads and exports what include/intfa.h
+declares, the ctypes mirror of the parameter block has the C layout, argument validation rejects bad
+blocks before any GPU call, and the Python entry points keep the reference's checks."""
+import ctypes
+import os
+import re
+import subprocess
+import tempfile
+
+import pytest
+import torch
+
+import int_flashattention_amd as M
+from int_flashattention_amd import _capi, _host
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "intfa.h")
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _capi.load()
+    text = open(HEADER).read()
+    declared = sorted(set(re.findall(r"^\s*(?:int|size_t|const char\*)\s+(intfa_\w+)\s*\(", text, flags=re.M)))
+    assert declared, "no declarations parsed from include/intfa.h"
+    assert set(declared) == set(_capi.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in intfa.h but not exported by libintfa.so"
+    assert lib.intfa_version() == 1
+    assert lib.intfa_block_n() == 128 == _host.BLOCK
+
+
+def test_ctypes_struct_matches_c_layout():
+    """Compiles a tiny C program against include/intfa.h and compares sizeof/offsetof with the ctypes mirror."""
+    fields = [f[0] for f in _capi.FwdParams._fields_]
+    body = "".join(f'printf("{f} %zu\\n", offsetof(intfa_fwd_params, {f}));\n' for f in fields)
+    src = f'#include <stdio.h>\n#include <stddef.h>\n#include "intfa.h"\nint main(void){{\n{body}printf("sizeof %zu\\n", sizeof(intfa_fwd_params));return 0;}}\n'
+    with tempfile.TemporaryDirectory() as td:
+        c = os.path.join(td, "layout.c"); exe = os.path.join(td, "layout")
+        open(c, "w").write(src)
+        subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), c, "-o", exe], check=True)
+        out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
+    got = dict(line.split() for line in out.strip().splitlines())
+    for f in fields:
+        assert int(got[f]) == getattr(_capi.FwdParams, f).offset, f
+    assert int(got["sizeof"]) == ctypes.sizeof(_capi.FwdParams)
+
+
+def _valid_block():
+    """A parameter block that passes validation (pointers are fake but aligned; it is never launched)."""
+    p = _capi.FwdParams()
+    for n in ("q", "k", "v", "out", "q_scale", "k_scale", "v_scale"):
+        setattr(p, n, 0x10000)
+    p.batch, p.heads, p.seqlen, p.head_dim = 1, 2, 256, 128
+    for t in ("q", "k", "v", "o"):
+        setattr(p, f"{t}_stride_b", 2 * 256 * 128); setattr(p, f"{t}_stride_h", 256 * 128); setattr(p, f"{t}_stride_n", 128)
+    p.qs_stride_b, p.qs_stride_h, p.qs_stride_n = 512, 256, 1
+    p.ks_stride_b, p.ks_stride_h, p.ks_stride_n = 512, 256, 1
+    p.vs_stride_b, p.vs_stride_h = 2, 1
+    p.sm_scale = 0.1
+    return p
+
+
+@pytest.mark.parametrize("mutate, code", [
+    (lambda p: setattr(p, "q", None), -1),
+    (lambda p: setattr(p, "v_scale", None), -1),
+    (lambda p: setattr(p, "head_dim", 48), -2),
+    (lambda p: setattr(p, "seqlen", 200), -3),
+    (lambda p: setattr(p, "seqlen", 0), -3),
+    (lambda p: setattr(p, "k", 0x10008), -4),
+    (lambda p: setattr(p, "q_stride_n", 120), -4),
+    (lambda p: setattr(p, "scale_dtype", 7), -5),
+    (lambda p: setattr(p, "io_dtype", 2), -5),
+    (lambda p: setattr(p, "num_splits", 4), -6),          # splits requested without a workspace
+    (lambda p: setattr(p, "batch", 0), -7),
+    (lambda p: (setattr(p, "num_splits", 65), setattr(p, "workspace", 0x10000), setattr(p, "workspace_bytes", 1 << 40)), -8),
+])
+def test_validation_rejects_bad_blocks_before_touching_the_gpu(mutate, code):
+    lib = _capi.load()
+    p = _valid_block()
+    mutate(p)
+    assert lib.intfa_fwd_full_int8(ctypes.byref(p), None) == code
+    assert lib.intfa_error_string(code).decode() not in ("", "ok")
+
+
+def test_null_block_and_error_strings():
+    lib = _capi.load()
+    assert lib.intfa_fwd_full_int8(None, None) == -1
+    assert lib.intfa_fwd_half_int8(None, None) == -1
+    assert lib.intfa_fwd_fp16(None, None) == -1
+    assert lib.intfa_error_string(0) == b"ok"
+    assert lib.intfa_error_string(700) == b"hip error"
+
+
+def test_workspace_query():
+    lib = _capi.load()
+    p = _valid_block()
+    assert lib.intfa_fwd_workspace_bytes(ctypes.byref(p)) == 0
+    p.num_splits = 4
+    rows = 4 * 1 * 2 * 256
+    assert lib.intfa_fwd_workspace_bytes(ctypes.byref(p)) == rows * 128 * 4 + rows * 4
+
+
+def test_entry_points_keep_the_reference_asserts():
+    q = torch.zeros((1, 1, 128, 48), dtype=torch.int8)
+    s = torch.ones((1, 1, 128), dtype=torch.float16)
+    with pytest.raises(AssertionError):                    # head dim not in {16, 32, 64, 128, 256}
+        _host.check_head_dims(q, q, q)
+    with pytest.raises(AssertionError):                    # q/k/v head dims differ
+        _host.check_head_dims(torch.zeros((1, 1, 128, 64)), torch.zeros((1, 1, 128, 32)), torch.zeros((1, 1, 128, 64)))
+    q = torch.zeros((1, 1, 128, 64), dtype=torch.int8)
+    with pytest.raises(RuntimeError, match="GPU only"):     # no CPU fallback
+        M.attention_full_int8(q, q, q, s, s, torch.ones((1, 1), dtype=torch.float16), False, 1.0)
+
+
+def test_package_quantisers_match_the_oracle():
+    import intfa_oracle as O
+    x = torch.randn((2, 3, 16, 32), generator=torch.Generator().manual_seed(0)).half()
+    for mine, ref in ((M.quant_pertoken, O.quant_pertoken), (M.quant_pertensor, O.quant_pertensor)):
+        a, sa = mine(x); b, sb = ref(x)
+        assert torch.equal(a, b) and torch.equal(sa, sb)

@@ -1,0 +1,286 @@
+"""Pins the CPU oracle (oracle/intfa_oracle.py) by means that do not retype its formulas: closed forms,
+invariants, special cases that reduce to library routines, and brute force on tiny inputs.
+
+The reference holds no golden vectors for the int8 paths (its single test asserts the fp16 forward with
+atol=1e-2, benchmark.py:242); that tolerance is used for the fp16 oracle below.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import intfa_oracle as O
+
+
+# ------------------------------------------------------------------------------------------ quantisers
+def test_quant_pertoken_invariants_and_bruteforce():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((2, 3, 5, 16), generator=g).half()
+    q, s = O.quant_pertoken(x)
+    assert q.dtype == torch.int8 and s.shape == (2, 3, 5) and s.dtype == torch.float16
+    assert int(q.abs().max()) == 127                      # every row reaches +-127
+    assert torch.all(q.abs().amax(dim=-1) == 127)
+    xn, sn = x.numpy(), s.numpy()
+    for idx in np.ndindex(2, 3, 5):                       # scalar restatement in numpy float16 arithmetic
+        row = xn[idx]
+        sc = np.float16(np.abs(row).max()) / np.float16(127)
+        assert sc == sn[idx]
+        for j in range(16):
+            want = int(np.rint(np.float16(row[j] / sc)))  # np.rint rounds half to even
+            assert want == int(q[idx][j])
+
+
+def test_quant_pertensor_one_scale_per_head():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn((2, 2, 8, 4), generator=g).half()
+    q, s = O.quant_pertensor(x)
+    assert s.shape == (2, 2)
+    for b in range(2):
+        for h in range(2):
+            assert float(s[b, h]) == float((x[b, h].abs().max() / 127))
+            assert int(q[b, h].abs().max()) == 127
+
+
+def test_mean_relative_error_matches_reference_definition():
+    a = torch.tensor([1.0, 2.0, 3.0, 4.0, 5.0, 6.0])
+    b = torch.tensor([1.0, 2.0, 3.3, 4.0, 5.0, 6.6])
+    # the reference looks at the last four elements only: |b-a| / (|b| + 1e-5)
+    want = np.mean([abs(3.3 - 3.0) / (3.3 + 1e-5), 0.0, 0.0, abs(6.6 - 6.0) / (6.6 + 1e-5)])
+    assert abs(O.mean_relative_error(a, b, calc_num=4) - want) < 1e-6
+    assert O.mean_relative_error(a, a) == 0.0
+
+
+# ------------------------------------------------------------------------------------------ integer parts
+def test_qk_int32_is_exact_integer_matmul():
+    g = torch.Generator().manual_seed(2)
+    q8 = torch.randint(-127, 128, (1, 2, 6, 8), generator=g, dtype=torch.int8)
+    k8 = torch.randint(-127, 128, (1, 2, 6, 8), generator=g, dtype=torch.int8)
+    s = O.qk_int32(q8, k8)
+    assert s.dtype == torch.int32
+    for h in range(2):
+        for i in range(6):
+            for j in range(6):
+                want = sum(int(q8[0, h, i, t]) * int(k8[0, h, j, t]) for t in range(8))
+                assert int(s[0, h, i, j]) == want
+    # extreme values at the largest head dim: |S| = 127*127*256 must survive the fp32 GEMM exactly
+    q8 = torch.full((1, 1, 2, 256), 127, dtype=torch.int8)
+    k8 = torch.full((1, 1, 2, 256), -127, dtype=torch.int8)
+    assert torch.all(O.qk_int32(q8, k8) == -127 * 127 * 256)
+    big = np.random.default_rng(0).integers(-127, 128, size=(2, 64, 256))
+    got = O.qk_int32(torch.tensor(big[None, :1], dtype=torch.int8), torch.tensor(big[None, 1:], dtype=torch.int8))
+    assert np.array_equal(got[0, 0].numpy().astype(np.int64), big[0].astype(np.int64) @ big[1].astype(np.int64).T)
+
+
+def test_p_requant_reference_exhaustive_over_fp16():
+    """Every fp16 value in [0, 1]: fp16(p)*127 -> fp16, +0.5 -> fp16, truncate (flash_atten_full_int8.py:49-51)."""
+    bits = np.arange(0, 0x3C01, dtype=np.uint16)          # 0.0 .. 1.0 inclusive
+    p = bits.view(np.float16)
+    got = O.p_requant_reference(torch.from_numpy(p.astype(np.float32))).numpy()
+    w = (p * np.float16(127)).astype(np.float16)           # numpy rounds each fp16 operation to fp16
+    u = (w + np.float16(0.5)).astype(np.float16)
+    want = np.trunc(u.astype(np.float32))
+    assert np.array_equal(got, want)
+    assert got.min() == 0 and got.max() == 127
+    # values between fp16 grid points are first rounded to fp16 (round-to-nearest-even)
+    x = torch.tensor([0.50006, 0.1234567, 0.99999, 1e-9])
+    got = O.p_requant_reference(x).numpy()
+    for v, gq in zip(x.numpy(), got):
+        hv = np.float16(v)
+        assert gq == np.trunc(np.float32(np.float16(np.float16(hv * np.float16(127)) + np.float16(0.5))))
+
+
+def test_p_requant_modes_differ_by_at_most_one():
+    p = torch.linspace(0, 1, 100001)
+    d = (O.p_requant_reference(p) - O.p_requant_rne(p)).abs()
+    assert d.max() <= 1
+
+
+# ------------------------------------------------------------------------------------------ online softmax
+def _dense_attention(x, v, causal):
+    """softmax over keys of logits x (already scaled, natural-log domain) times v, all fp32, torch.softmax."""
+    if causal:
+        n = x.shape[-1]
+        x = x.masked_fill(~torch.tril(torch.ones((n, n), dtype=torch.bool)), float("-inf"))
+    return torch.softmax(x, dim=-1) @ v
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_fp_variant_reduces_to_torch_softmax_for_any_block(causal):
+    q, k, v, _ = O.make_inputs(1, 2, 64, 16, seed=3, std=0.5)
+    sm = 0.3
+    want = _dense_attention((q.float() @ k.float().transpose(2, 3)) * sm, v.float(), causal)
+    for bm, bn in ((64, 64), (32, 16), (16, 16), (64, 8)):
+        got, lse = O.attention_fp(q, k, v, causal, sm, block_m=bm, block_n=bn, return_lse=True)
+        # P is rounded to fp16 before PV (flash_atten_fp.py:54); the reference's own tolerance is atol=1e-2
+        assert (got.float() - want).abs().max() < 2e-3
+        x = (q.float() @ k.float().transpose(2, 3)) * sm
+        if causal:
+            x = x.masked_fill(~torch.tril(torch.ones((64, 64), dtype=torch.bool)), float("-inf"))
+        want_lse = torch.logsumexp(x, dim=-1) * O.LOG2E      # M = m + log2(l) is the base-2 log-sum-exp
+        assert (lse - want_lse).abs().max() < 1e-4
+
+
+def test_half_variant_dense_special_case():
+    """Half-int8 with block_n = N is dequantise -> torch.softmax -> fp16(P) @ V."""
+    q, k, v, _ = O.make_inputs(1, 2, 32, 16, seed=4)
+    q8, qs = O.quant_pertoken(q)
+    k8, ks = O.quant_pertoken(k)
+    sm = 0.25
+    x = (q8.float() @ k8.float().transpose(2, 3)) * qs.float()[..., None] * ks.float()[:, :, None, :]
+    pm = torch.softmax(x * sm, dim=-1)
+    got = O.attention_int8(q8, k8, v, qs, ks, False, sm, block_m=32, block_n=32)
+    # oracle rounds the UNNORMALISED p (<= 1) to fp16 and divides by l afterwards
+    want = pm @ v.float()
+    assert (got.float() - want).abs().max() < 2e-3
+    for bn in (8, 16):
+        other = O.attention_int8(q8, k8, v, qs, ks, False, sm, block_m=32, block_n=bn)
+        assert (other.float() - got.float()).abs().max() < 2e-3
+
+
+def test_full_int8_unit_scales_is_integer_attention_bruteforce():
+    """All scales one, tiny integers: evaluate the reference loop with Python scalars for one head."""
+    g = torch.Generator().manual_seed(5)
+    N, D, BN = 4, 2, 2
+    q8 = torch.randint(-3, 4, (1, 1, N, D), generator=g, dtype=torch.int8)
+    k8 = torch.randint(-3, 4, (1, 1, N, D), generator=g, dtype=torch.int8)
+    v8 = torch.randint(-127, 128, (1, 1, N, D), generator=g, dtype=torch.int8)
+    one = torch.ones((1, 1, N), dtype=torch.float16)
+    vs = torch.ones((1, 1), dtype=torch.float16)
+    sm = 0.5
+    got = O.attention_full_int8(q8, k8, v8, one, one, vs, False, sm, block_m=2, block_n=BN).float()[0, 0]
+    c = np.float32(sm) * np.float32(O.LOG2E)
+    for i in range(N):
+        m, l, acc = -math.inf, 1.0, [0.0] * D
+        for j0 in range(0, N, BN):
+            s = [sum(int(q8[0, 0, i, t]) * int(k8[0, 0, j, t]) for t in range(D)) for j in range(j0, j0 + BN)]
+            m_new = max(m, max(np.float32(x) * c for x in s))
+            p = [float(np.exp2(np.float32(np.float32(x) * c - np.float32(m_new)))) for x in s]
+            p8 = [int(np.trunc(np.float32(np.float16(np.float16(np.float16(x) * np.float16(127)) + np.float16(0.5))))) for x in p]
+            alpha = float(np.exp2(np.float32(m - m_new))) if m != -math.inf else 0.0
+            l = l * alpha + sum(p)
+            for t in range(D):
+                tmp = sum(p8[jj] * int(v8[0, 0, j0 + jj, t]) for jj in range(BN))
+                acc[t] = acc[t] * alpha + tmp * 1.0 / 127
+            m = m_new
+        for t in range(D):
+            assert abs(got[i, t].item() - acc[t] / l) <= 1e-3 * max(1.0, abs(acc[t] / l))
+
+
+def test_full_int8_constant_v_gives_quantised_mass_ratio():
+    """V8 == c everywhere: O = c * v_scale * sum(P8) / (127 * l); with one key block sum(P8) and l are dense."""
+    q, k, _, _ = O.make_inputs(1, 1, 16, 8, seed=6)
+    q8, qs = O.quant_pertoken(q)
+    k8, ks = O.quant_pertoken(k)
+    v8 = torch.full((1, 1, 16, 8), 100, dtype=torch.int8)
+    vs = torch.tensor([[0.02]], dtype=torch.float16)
+    sm = 0.35
+    got = O.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, block_m=16, block_n=16).float()
+    x = (q8.float() @ k8.float().transpose(2, 3)) * qs.float()[..., None] * ks.float()[:, :, None, :] * (sm * O.LOG2E)
+    p = torch.exp2(x - x.max(dim=-1, keepdim=True).values)
+    ratio = O.p_requant_reference(p).sum(-1) / (127 * p.sum(-1))
+    want = 100 * float(vs) * ratio
+    assert (got - want[..., None]).abs().max() < 2e-3
+    assert 0.9 < ratio.mean() < 1.1
+
+
+def test_l_sums_unquantised_p():
+    """Rows whose probabilities all fall below 1/254 quantise to P8 == 0: the numerator vanishes, l does not."""
+    N = 512
+    q8 = torch.zeros((1, 1, N, 8), dtype=torch.int8)          # all logits equal -> p = 1 for the first block ...
+    q8[..., 0] = 1
+    k8 = torch.zeros((1, 1, N, 8), dtype=torch.int8)
+    k8[0, 0, 0, 0] = 127                                       # ... except key 0 dominates by a wide margin
+    v8 = torch.full((1, 1, N, 8), 50, dtype=torch.int8)
+    v8[0, 0, 0] = 0
+    one = torch.ones((1, 1, N), dtype=torch.float16)
+    vs = torch.ones((1, 1), dtype=torch.float16)
+    got = O.attention_full_int8(q8, k8, v8, one, one, vs, False, 0.1, block_m=N, block_n=N).float()
+    # logits: key0 = 12.7, others 0 -> p_others = exp(-12.7) ~ 3e-6 each, P8 = 0; key 0 has V = 0
+    assert torch.all(got == 0)
+    exact = O.attention_exact(q8.half(), k8.half(), v8.half(), False, 0.1).float()
+    assert exact.abs().max() > 0                               # the unquantised path keeps a little mass
+
+
+@pytest.mark.parametrize("variant", ["full", "half"])
+def test_causal_equals_dense_masked_evaluation(variant):
+    q, k, v, _ = O.make_inputs(1, 2, 64, 16, seed=7)
+    q8, qs = O.quant_pertoken(q)
+    k8, ks = O.quant_pertoken(k)
+    v8, vs = O.quant_pertensor(v)
+    sm = 0.25
+    x = (q8.float() @ k8.float().transpose(2, 3)) * qs.float()[..., None] * ks.float()[:, :, None, :]
+    if variant == "half":
+        got = O.attention_int8(q8, k8, v, qs, ks, True, sm, block_m=32, block_n=16).float()
+        want = _dense_attention(x * sm, v.float(), True)
+        tol = 2e-3
+    else:
+        got = O.attention_full_int8(q8, k8, v8, qs, ks, vs, True, sm, block_m=32, block_n=16).float()
+        want = _dense_attention(x * sm, v8.float() * vs.float()[..., None, None], True)
+        tol = 3e-2                                             # P8 has 1/127 resolution
+    assert (got - want).abs().max() < tol
+    # row 0 attends to key 0 only
+    first = v.float()[:, :, 0] if variant == "half" else v8.float()[:, :, 0] * vs.float()[..., None]
+    assert (got[:, :, 0] - first).abs().max() < 1e-2
+    # a causal run never looks at keys above the diagonal: perturbing them changes nothing
+    k8b = k8.clone(); k8b[:, :, 40:] = 0
+    vb = v.clone(); vb[:, :, 40:] = 0
+    v8b = v8.clone(); v8b[:, :, 40:] = 0
+    if variant == "half":
+        again = O.attention_int8(q8, k8b, vb, qs, ks, True, sm, block_m=32, block_n=16).float()
+    else:
+        again = O.attention_full_int8(q8, k8b, v8b, qs, ks, vs, True, sm, block_m=32, block_n=16).float()
+    assert torch.equal(again[:, :, :40], got[:, :, :40])
+
+
+def test_block_n_dependence_is_bounded_but_real():
+    """P is quantised against the running maximum, so block_n changes the result a little (not zero)."""
+    q, k, v, _ = O.make_inputs(1, 2, 256, 64, seed=8)
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    a = O.attention_full_int8(q8, k8, v8, qs, ks, vs, False, 0.125, block_n=128).float()
+    b = O.attention_full_int8(q8, k8, v8, qs, ks, vs, False, 0.125, block_n=64).float()
+    d = (a - b).abs().max().item()
+    assert 0 < d < 2e-2
+
+
+# ------------------------------------------------------------------------------------------ split-KV
+def test_splitkv_combine_reproduces_dense_softmax():
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn((1, 2, 8, 24), generator=g) * 3           # logits, natural-log domain
+    v = torch.randn((1, 2, 24, 4), generator=g)
+    want = torch.softmax(x, dim=-1) @ v
+    parts, lses = [], []
+    for lo, hi in ((0, 8), (8, 16), (16, 24), (24, 24)):       # the last split is empty
+        if lo == hi:
+            parts.append(torch.zeros((1, 2, 8, 4))); lses.append(torch.full((1, 2, 8), float("-inf")))
+            continue
+        xs = x[..., lo:hi]
+        parts.append(torch.softmax(xs, dim=-1) @ v[:, :, lo:hi])
+        lses.append(torch.logsumexp(xs, dim=-1) * O.LOG2E)
+    got, lse = O.splitkv_combine(torch.stack(parts), torch.stack(lses))
+    assert (got - want).abs().max() < 1e-5
+    assert (lse - torch.logsumexp(x, dim=-1) * O.LOG2E).abs().max() < 1e-4
+
+
+def test_splitkv_ranges_follow_ceil_partition():
+    assert O.splitkv_ranges(1024, 128, 3) == [(0, 3), (3, 6), (6, 8)]
+    assert O.splitkv_ranges(256, 128, 4) == [(0, 1), (1, 2), (2, 2), (3, 2)]
+    assert O.splitkv_ranges(512, 128, 1) == [(0, 4)]
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_full_int8_split_agrees_with_single_pass(causal):
+    q, k, v, _ = O.make_inputs(1, 2, 256, 32, seed=10)
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    one = O.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, 0.2, block_m=64, block_n=64).float()
+    same = O.attention_full_int8_splitkv(q8, k8, v8, qs, ks, vs, causal, 0.2, 1, block_m=64, block_n=64).float()
+    assert (one - same).abs().max() < 1e-3                     # one split: identical up to the fp16 store
+    two = O.attention_full_int8_splitkv(q8, k8, v8, qs, ks, vs, causal, 0.2, 2, block_m=64, block_n=64).float()
+    assert (one - two).abs().max() < 2e-2                      # later splits quantise P against their own maximum
+
+
+def test_exact_attention_matches_reference_recipe():
+    q, k, v, _ = O.make_inputs(1, 1, 16, 8, seed=11, std=0.5)
+    got = O.attention_exact(q, k, v, True, 1.0).float()
+    want = _dense_attention(q.float() @ k.float().transpose(2, 3), v.float(), True)
+    assert (got - want).abs().max() < 2e-3
