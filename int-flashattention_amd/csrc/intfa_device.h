@@ -105,17 +105,25 @@ __device__ __forceinline__ TileLoadLane<ROW_BYTES, IS_V> tile_load_lane(uint32_t
     }
     return t;
 }
+#if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
+// The global side is addressed through a buffer resource (base pointer of the (batch, head) slice in SGPRs)
+// plus a wave-uniform byte offset in an SGPR plus the lane's 32-bit offset: no 64-bit per-lane pointers.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
 template <int ROW_BYTES, bool IS_V>
-__device__ __forceinline__ void issue_tile_load(const char* gtile, uint32_t row_stride, char* lds_tile, int wave,
-                                                const TileLoadLane<ROW_BYTES, IS_V>& ln) {
+__device__ __forceinline__ void issue_tile_load(__amdgpu_buffer_rsrc_t rsrc, uint32_t tile_off, uint32_t row_stride,
+                                                char* lds_tile, int wave, const TileLoadLane<ROW_BYTES, IS_V>& ln) {
     using T = TileLoadLane<ROW_BYTES, IS_V>;
 #pragma unroll
     for (int it = 0; it < T::NINST / 4; ++it) {
         const int i = it * 4 + wave;                 // wave-uniform instruction index
-        const char* g = gtile + (uint64_t)(i * T::RPI) * row_stride;
-        __builtin_amdgcn_global_load_lds(INTFA_GLB(g + ln.off[it % T::NV]), INTFA_LDS(lds_tile + i * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)INTFA_LDS(lds_tile + i * 1024), 16,
+                                                 ln.off[it % T::NV], tile_off + (uint32_t)(i * T::RPI) * row_stride, 0, 0);
     }
 }
+
+#endif  // __HIP_DEVICE_COMPILE__
 
 __device__ __forceinline__ float wave_half_swap(float x) {      // value held by lane l ^ 32
     return __shfl_xor(x, 32);

@@ -14,6 +14,8 @@ namespace intfa {
 
 enum { VAR_FULL = 0, VAR_HALF = 1 };
 
+template <bool V> struct BoolTag { static constexpr bool value = V; };
+
 template <int D> struct SmemInt8 {
     char k[2][kBlockN * D];
     char v[2][kBlockN * D * 2];     // sized for 16-bit V; the int8 variant uses the first half of each
@@ -23,6 +25,7 @@ template <int D> struct SmemInt8 {
 // One workgroup = one (batch, head, 128-query block[, split]).
 template <int VARIANT, int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUMP_S, bool SPLIT>
 __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T (32 bytes of head_dim each)
     constexpr int DT = D / 32;                   // 32-wide output tiles along head_dim
     constexpr int VB = (VARIANT == VAR_FULL) ? 1 : 2;   // bytes per V element
@@ -98,39 +101,56 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
     const int g16 = lane >> 4, i16 = lane & 15, jj = i16 >> 1;
     const int v_row0 = 8 * (jj >> 2) + 4 * lh + (jj & 3);          // + 16*w + 32*st
     const int v_sub = 8 * (i16 & 1);
+    const int v_swz = swz_v<VROW>(v_row0) & ((VROW / 16 < 8 ? VROW / 16 : 8) - 1);
 
     const auto k_lane = tile_load_lane<D, false>((uint32_t)p.k_sn, wave, lane);
     const auto v_lane = tile_load_lane<VROW, true>((uint32_t)p.v_sn, wave, lane);
-    auto issue_loads = [&](int nb, char* dK, char* dV) {
-        issue_tile_load<D, false>(Kg + (int64_t)nb * kBlockN * p.k_sn, (uint32_t)p.k_sn, dK, wave, k_lane);
-        if (!DUMP_S) issue_tile_load<VROW, true>(Vg + (int64_t)nb * kBlockN * p.v_sn, (uint32_t)p.v_sn, dV, wave, v_lane);
+    const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen - 1) * p.k_sn + D));
+    const __amdgpu_buffer_rsrc_t v_rsrc = make_rsrc(DUMP_S ? Kg : Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + VROW));
+    auto issue_loads = [&](int nb, char* dK, char* dV) __attribute__((always_inline)) {
+        issue_tile_load<D, false>(k_rsrc, (uint32_t)(nb * kBlockN) * (uint32_t)p.k_sn, (uint32_t)p.k_sn, dK, wave, k_lane);
+        if (!DUMP_S) issue_tile_load<VROW, true>(v_rsrc, (uint32_t)(nb * kBlockN) * (uint32_t)p.v_sn, (uint32_t)p.v_sn, dV, wave, v_lane);
     };
-    const uint32_t ks_lane = (uint32_t)tid * (uint32_t)p.ks_sn;
-    auto load_ks = [&](int nb) -> float {
-        if (DUMP_S || tid >= kBlockN) return 0.f;
-        const int64_t base = ks_base + (int64_t)nb * kBlockN * p.ks_sn;     // wave-uniform
-        if (p.scale_dtype == 0) return (float)((const _Float16*)Ksg + base)[ks_lane];
-        if (p.scale_dtype == 1) return __builtin_bit_cast(float, ((uint32_t)((const uint16_t*)Ksg + base)[ks_lane]) << 16);
-        return ((const float*)Ksg + base)[ks_lane];
+    // k_scale of the block: thread t < 128 fetches the scale of key t, converted to fp32 when stored to LDS
+    const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
+    const __amdgpu_buffer_rsrc_t ks_rsrc =
+        make_rsrc(DUMP_S ? Kg : Ksg + ks_base * ks_esize, DUMP_S ? 0u : (uint32_t)(((p.seqlen - 1) * p.ks_sn + 1) * ks_esize));
+    const uint32_t ks_lane = (uint32_t)(tid & (kBlockN - 1)) * (uint32_t)(p.ks_sn * ks_esize);
+    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {           // raw bits; converted by cvt_ks
+        if (DUMP_S) return 0u;
+        const uint32_t so = (uint32_t)(nb * kBlockN) * (uint32_t)(p.ks_sn * ks_esize);
+        if (p.scale_dtype == 2) return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ks_rsrc, ks_lane, so, 0);
+        return (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(ks_rsrc, ks_lane, so, 0);
+    };
+    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float {
+        if (p.scale_dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+        if (p.scale_dtype == 1) return __builtin_bit_cast(float, raw << 16);
+        return __builtin_bit_cast(float, raw);
     };
 
-    auto compute = [&](int nb, const char* cK, const char* cV, const float* cKs) {
-        const bool diag = CAUSAL && (nb == mb);
+    // One key block.  DIAG selects the code for the block on the causal diagonal (mask + sub-tile skip).
+    auto compute = [&](auto diag_tag, int nb, const char* cK, const char* cV, const float* cKs) __attribute__((always_inline)) {
+        constexpr bool DIAG = decltype(diag_tag)::value;
+        // Loop-invariant address pieces are re-derived per block from two opaque values, so the compiler does not
+        // keep a register per (k-step, d-tile) variant alive across the whole loop.
+        int ksw = k_swz, vsw = v_swz;
+        asm volatile("" : "+v"(ksw), "+v"(vsw));
         // -------- pass 1: S^T sub-tiles, dequantise by k_scale, running row max
         float t[4][16];
         float mx = -INFINITY;
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
-            if (CAUSAL && diag && st > wave) {               // sub-tile entirely above the diagonal
+            if (DIAG && st > wave) {                          // sub-tile entirely above the diagonal
 #pragma unroll
                 for (int r = 0; r < 16; ++r) t[st][r] = -INFINITY;
                 continue;
             }
+            __builtin_amdgcn_sched_barrier(0);
             v16i acc = {0};
             const char* krow = cK + (32 * st + lq) * D;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const v4i a = *(const v4i*)(krow + (((2 * ks + lh) ^ k_swz) << 4));
+                const v4i a = *(const v4i*)(krow + (((2 * ks + lh) ^ ksw) << 4));
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qreg[ks], acc, 0, 0, 0);
             }
             if (DUMP_S) {
@@ -144,9 +164,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
 #pragma unroll
                 for (int b4 = 0; b4 < 4; ++b4) {
                     float x = (float)acc[4 * a4 + b4] * kk[b4];
-                    if (CAUSAL && diag && st == wave) {
-                        const int key = 8 * a4 + 4 * lh + b4;       // position inside the 32x32 diagonal tile
-                        if (key > lq) x = -INFINITY;
+                    if (DIAG) {
+                        // position of the key inside the 32x32 tile on the diagonal vs this lane's query
+                        if (st == wave && (8 * a4 + b4) > lq - 4 * lh) x = -INFINITY;
                     }
                     t[st][4 * a4 + b4] = x;
                     mx = fmaxf(mx, x);
@@ -165,6 +185,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
             const float bias = (PROUND == 0 ? kLog2_127 : 0.f) - m_new;
 #pragma unroll
             for (int st = 0; st < 4; ++st) {
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int w4 = 0; w4 < 4; ++w4) {
                     unsigned pk = 0;
@@ -192,18 +213,19 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
                 }
             }
             // -------- P V on int8 MFMA: O^T[d, q] += V^T[d, key] P^T[key, q]
+            const char* vbase = cV + v_row0 * VROW + v_sub;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
+                __builtin_amdgcn_sched_barrier(0);
                 v16i acc = {0};
+                const int coff = ((2 * dt + (g16 & 1)) ^ vsw) << 4;
 #pragma unroll
                 for (int st = 0; st < 4; ++st) {
-                    if (CAUSAL && diag && st > wave) continue;
-                    const int c = 2 * dt + (g16 & 1);
-                    const int r0 = 32 * st + v_row0, r1 = r0 + 16;
+                    if (DIAG && st > wave) continue;
                     const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                        (__attribute__((address_space(3))) v2i*)INTFA_LDS(cV + r0 * VROW + ((c ^ swz_v<VROW>(r0)) << 4) + v_sub));
+                        (__attribute__((address_space(3))) v2i*)INTFA_LDS(vbase + (32 * st) * VROW + coff));
                     const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                        (__attribute__((address_space(3))) v2i*)INTFA_LDS(cV + r1 * VROW + ((c ^ swz_v<VROW>(r1)) << 4) + v_sub));
+                        (__attribute__((address_space(3))) v2i*)INTFA_LDS(vbase + (32 * st + 16) * VROW + coff));
                     const v4i a = {lo[0], lo[1], hi[0], hi[1]};
                     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, p8[st], acc, 0, 0, 0);
                 }
@@ -213,28 +235,41 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
         }
         l_run = fmaf(l_run, alpha, lsum);
     };
+    // One pipeline step on LDS buffer BUF: wait for this block's tiles (issued one step earlier), make them
+    // visible to all four waves, start the copy of the next block into the other buffer, compute.
+    auto step = [&](auto buf_tag, auto diag_tag, int nb) __attribute__((always_inline)) {
+        constexpr bool B1 = decltype(buf_tag)::value;
+        char* cK = B1 ? sK1 : sK0; char* cV = B1 ? sV1 : sV0; float* cKs = B1 ? sKs1 : sKs0;
+        char* nK = B1 ? sK0 : sK1; char* nV = B1 ? sV0 : sV1; float* nKs = B1 ? sKs0 : sKs1;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const bool more = nb + 1 < nb_end;
+        uint32_t ks_next = 0;
+        if (more) { issue_loads(nb + 1, nK, nV); ks_next = load_ks(nb + 1); }
+        compute(diag_tag, nb, cK, cV, cKs);
+        if (more && tid < kBlockN) nKs[tid] = cvt_ks(ks_next);
+    };
 
-    // ---- main loop: K/V tiles double-buffered in LDS, one barrier per key block
+    // ---- main loop: K/V tiles double-buffered in LDS, one barrier per key block.  The block on the causal
+    // diagonal is always the last of the range and gets its own code instance after the loop.
     if (nb_begin < nb_end) {
         issue_loads(nb_begin, sK0, sV0);
         {
-            const float s0 = load_ks(nb_begin);
-            if (tid < kBlockN) sKs0[tid] = s0;
+            const uint32_t s0 = load_ks(nb_begin);
+            if (tid < kBlockN) sKs0[tid] = cvt_ks(s0);
         }
-        for (int nb = nb_begin; nb < nb_end; nb += 2) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
-            float ks_next = 0.f;
-            if (nb + 1 < nb_end) { issue_loads(nb + 1, sK1, sV1); ks_next = load_ks(nb + 1); }
-            compute(nb, sK0, sV0, sKs0);
-            if (nb + 1 < nb_end) {
-                if (tid < kBlockN) sKs1[tid] = ks_next;
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();
-                if (nb + 2 < nb_end) { issue_loads(nb + 2, sK0, sV0); ks_next = load_ks(nb + 2); }
-                compute(nb + 1, sK1, sV1, sKs1);
-                if (nb + 2 < nb_end && tid < kBlockN) sKs0[tid] = ks_next;
-            }
+        const bool has_diag = CAUSAL && (nb_end == mb + 1);
+        const int plain_end = has_diag ? nb_end - 1 : nb_end;
+        int nb = nb_begin;
+        while (true) {
+            if (nb >= plain_end) break;
+            step(BoolTag<false>{}, BoolTag<false>{}, nb++);
+            if (nb >= plain_end) break;
+            step(BoolTag<true>{}, BoolTag<false>{}, nb++);
+        }
+        if (CAUSAL && has_diag) {
+            if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb);
+            else step(BoolTag<true>{}, BoolTag<true>{}, nb);
         }
     }
     if (DUMP_S) return;
@@ -290,6 +325,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
             }
         }
     if (p.lse != nullptr && lh == 0) p.lse[((int64_t)(b * p.heads) + h) * p.seqlen + q_row] = lse;
+#endif  // __HIP_DEVICE_COMPILE__
 }
 
 }  // namespace intfa
