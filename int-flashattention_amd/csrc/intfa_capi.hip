@@ -101,10 +101,10 @@ int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t str
 }
 
 // Expands the runtime switches (head_dim, causal, out dtype, P rounding, split) into template arguments.
-template <int VARIANT> int dispatch_int8(const intfa_fwd_params* p, const KParams& kp, hipStream_t stream) {
+int dispatch_full_int8(const intfa_fwd_params* p, const KParams& kp, hipStream_t stream) {
     const bool causal = kp.causal != 0, bf = p->io_dtype == INTFA_BF16, split = kp.num_splits > 1;
-    const int pr = (VARIANT == VAR_FULL && p->p_round == INTFA_PROUND_REFERENCE) ? 1 : 0;
-#define INTFA_L(DD, C, O, PR, SP) return launch(fwd_int8_kernel<VARIANT, DD, C, O, PR, false, SP>, kp, stream)
+    const int pr = (p->p_round == INTFA_PROUND_REFERENCE) ? 1 : 0;
+#define INTFA_L(DD, C, O, PR, SP) return launch(fwd_full_int8_kernel<DD, C, O, PR, false, SP>, kp, stream)
 #define INTFA_SW_SP(DD, C, O, PR) do { if (split) INTFA_L(DD, C, O, PR, true); else INTFA_L(DD, C, O, PR, false); } while (0)
 #define INTFA_SW_PR(DD, C, O) do { if (pr) INTFA_SW_SP(DD, C, O, 1); else INTFA_SW_SP(DD, C, O, 0); } while (0)
 #define INTFA_SW_O(DD, C) do { if (bf) INTFA_SW_PR(DD, C, 1); else INTFA_SW_PR(DD, C, 0); } while (0)
@@ -153,7 +153,7 @@ int intfa_fwd_full_int8(const intfa_fwd_params* p, void* stream) {
     if (p->p_round != INTFA_PROUND_RNE && p->p_round != INTFA_PROUND_REFERENCE) return INTFA_ERR_DTYPE;
     rc = setup_split(p, &kp);
     if (rc != INTFA_OK) return rc;
-    rc = dispatch_int8<VAR_FULL>(p, kp, (hipStream_t)stream);
+    rc = dispatch_full_int8(p, kp, (hipStream_t)stream);
     if (rc != INTFA_OK || kp.num_splits <= 1) return rc;
     return launch_combine(p, kp, (hipStream_t)stream);
 }
@@ -187,8 +187,8 @@ int intfa_debug_qk_int32(const intfa_fwd_params* p, int32_t* s_out, void* stream
     kp.causal = 0;
     kp.scale_dtype = INTFA_F32;
     switch (kp.head_dim) {
-        case 64: return launch(fwd_int8_kernel<VAR_FULL, 64, false, 0, 0, true, false>, kp, (hipStream_t)stream);
-        case 128: return launch(fwd_int8_kernel<VAR_FULL, 128, false, 0, 0, true, false>, kp, (hipStream_t)stream);
+        case 64: return launch(fwd_full_int8_kernel<64, false, 0, 0, true, false>, kp, (hipStream_t)stream);
+        case 128: return launch(fwd_full_int8_kernel<128, false, 0, 0, true, false>, kp, (hipStream_t)stream);
     }
     return INTFA_ERR_HEAD_DIM;
 }

@@ -68,7 +68,7 @@ __device__ __forceinline__ float load_scale(const char* base, int64_t idx, int d
 // that the 8 rows touched together by one group of lanes fall into 8 different bank groups.
 // K rows are read by 8 consecutive lanes as 8 consecutive rows.
 template <int ROW_BYTES> __device__ __forceinline__ int swz_k(int row) {
-    if (ROW_BYTES >= 128) return row & 7;
+    if (ROW_BYTES >= 128) return (row & 7) ^ ((row >> 3) & 1);   // 16 consecutive rows -> 16 distinct 16-byte bank groups
     return (row >> 1) & 3;                       // 64-byte rows: two rows share a 128-byte line
 }
 // V rows are read by the transposing load as rows {0,1,2,3,8,9,10,11} + 4h of a 32-key sub-tile.
@@ -105,28 +105,56 @@ __device__ __forceinline__ TileLoadLane<ROW_BYTES, IS_V> tile_load_lane(uint32_t
     }
     return t;
 }
-#if defined(__HIP_DEVICE_COMPILE__)   // buffer-resource builtins exist in the device pass only
-// The global side is addressed through a buffer resource (base pointer of the (batch, head) slice in SGPRs)
-// plus a wave-uniform byte offset in an SGPR plus the lane's 32-bit offset: no 64-bit per-lane pointers.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+// The global side is addressed through a buffer resource (base pointer of the (batch, head) slice, SGPRs) plus a
+// wave-uniform byte offset (SGPR) plus the lane's 32-bit offset: no 64-bit per-lane pointers.  The copy itself is
+// written as inline assembly (M0 = LDS destination of the wave's 1 KiB, then buffer_load_dwordx4 ... lds) so that
+// the compiler does not serialise later LDS reads of the OTHER buffer behind it; completion is awaited explicitly
+// with s_waitcnt vmcnt(0) before the workgroup barrier that publishes the tile.
+__device__ __forceinline__ v4i make_rsrc(const void* base, uint32_t bytes) {
+    const uint64_t a = (uint64_t)base;
+    v4i r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+    r[1] = __builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu));   // stride 0: raw buffer
+    r[2] = __builtin_amdgcn_readfirstlane((int)bytes);                              // num_records, bounds-checked
+    r[3] = 0x00020000;
+    return r;
+}
+// Issues wave instruction number `it` (0 .. NINST/4 - 1) of this wave's share of one tile copy.
+template <int ROW_BYTES, bool IS_V>
+__device__ __forceinline__ void issue_tile_part(v4i rsrc, uint32_t tile_off, uint32_t row_stride, uint32_t lds_tile,
+                                                int wave, const TileLoadLane<ROW_BYTES, IS_V>& ln, int it) {
+    using T = TileLoadLane<ROW_BYTES, IS_V>;
+    const int i = it * 4 + wave;                     // wave-uniform instruction index
+    const uint32_t m0v = lds_tile + (uint32_t)i * 1024u;
+    const uint32_t soff = tile_off + (uint32_t)(i * T::RPI) * row_stride;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(m0v), "v"(ln.off[it % T::NV]), "s"(rsrc), "s"(soff) : "memory");
 }
 template <int ROW_BYTES, bool IS_V>
-__device__ __forceinline__ void issue_tile_load(__amdgpu_buffer_rsrc_t rsrc, uint32_t tile_off, uint32_t row_stride,
-                                                char* lds_tile, int wave, const TileLoadLane<ROW_BYTES, IS_V>& ln) {
+__device__ __forceinline__ void issue_tile_load(v4i rsrc, uint32_t tile_off, uint32_t row_stride, uint32_t lds_tile,
+                                                int wave, const TileLoadLane<ROW_BYTES, IS_V>& ln) {
     using T = TileLoadLane<ROW_BYTES, IS_V>;
 #pragma unroll
-    for (int it = 0; it < T::NINST / 4; ++it) {
-        const int i = it * 4 + wave;                 // wave-uniform instruction index
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)INTFA_LDS(lds_tile + i * 1024), 16,
-                                                 ln.off[it % T::NV], tile_off + (uint32_t)(i * T::RPI) * row_stride, 0, 0);
-    }
+    for (int it = 0; it < T::NINST / 4; ++it) issue_tile_part<ROW_BYTES, IS_V>(rsrc, tile_off, row_stride, lds_tile, wave, ln, it);
 }
 
-#endif  // __HIP_DEVICE_COMPILE__
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {   // round-to-nearest-even
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
 
-__device__ __forceinline__ float wave_half_swap(float x) {      // value held by lane l ^ 32
-    return __shfl_xor(x, 32);
+// Reductions across the two lanes that share a query column (lane l and lane l ^ 32): v_permlane32_swap turns
+// one register into (lower halves, upper halves), so one swap plus one max/add serves all 64 lanes.
+__device__ __forceinline__ float half_pair_max(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+}
+__device__ __forceinline__ float half_pair_sum(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

@@ -1,42 +1,38 @@
-// Forward kernels with int8 Q K^T: full-int8 (int8 P V) and half-int8 (fp16/bf16 P V).
+// Forward kernel with int8 Q K^T and int8 P V (full-int8).
 //
-// Algorithm restated from the reference tile loop (flash_atten_full_int8.py:9-71, flash_atten_int8.py:9-66):
-// per key block of kBlockN keys, S = Q8 K8^T in int32; X = S * q_scale[row] * k_scale[col]; running max m in
-// the exp2 domain; P = exp2(X * c - m_new); l sums the UNQUANTISED P; P is requantised to int8 with the fixed
-// scale 127 (full) or cast to half precision (half); acc = acc * alpha + P V; output acc / l.
+// Algorithm restated from the reference tile loop (flash_atten_full_int8.py:9-71): per key block of kBlockN
+// keys, S = Q8 K8^T in int32; X = S * q_scale[row] * k_scale[col]; running max m in the exp2 domain;
+// P = exp2(X * c - m_new); l sums the UNQUANTISED P; P is requantised to int8 with the fixed scale 127;
+// acc = acc * alpha + P8 V8; output acc * v_scale / (127 l).
 // Differences in evaluation order that stay within fp32 rounding: q_scale * c is folded into one per-row
 // factor, v_scale / 127 is applied once in the epilogue, and (RNE mode) the factor 127 is folded into the
 // exponent as exp2(x + log2 127).
+//
+// One workgroup (4 waves) owns 128 query rows of one (batch, head); wave w owns rows 32w..32w+31.
+// LDS holds two K tiles, two V tiles and two k_scale vectors (double buffering); all LDS traffic uses
+// integer offsets into ONE array so that operand addresses are a lane register plus an immediate.
 #pragma once
 #include "intfa_device.h"
 
 namespace intfa {
 
-enum { VAR_FULL = 0, VAR_HALF = 1 };
-
 template <bool V> struct BoolTag { static constexpr bool value = V; };
 
-template <int D> struct SmemInt8 {
-    char k[2][kBlockN * D];
-    char v[2][kBlockN * D * 2];     // sized for 16-bit V; the int8 variant uses the first half of each
-    float ks[2][kBlockN];
-};
-
-// One workgroup = one (batch, head, 128-query block[, split]).
-template <int VARIANT, int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUMP_S, bool SPLIT>
-__global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) {
+template <int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUMP_S, bool SPLIT>
+__global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T (32 bytes of head_dim each)
     constexpr int DT = D / 32;                   // 32-wide output tiles along head_dim
-    constexpr int VB = (VARIANT == VAR_FULL) ? 1 : 2;   // bytes per V element
-    constexpr int VROW = D * VB;
-
-    __shared__ __attribute__((aligned(1024))) char sK0[kBlockN * D];
-    __shared__ __attribute__((aligned(1024))) char sK1[kBlockN * D];
-    __shared__ __attribute__((aligned(1024))) char sV0[kBlockN * VROW];
-    __shared__ __attribute__((aligned(1024))) char sV1[kBlockN * VROW];
-    __shared__ __attribute__((aligned(16))) float sKs0[kBlockN];
-    __shared__ __attribute__((aligned(16))) float sKs1[kBlockN];
+    constexpr int NST = kBlockN / 32;            // 32-key sub-tiles per key block
+    constexpr int KT = kBlockN * D;              // bytes of one K tile (and of one int8 V tile)
+    constexpr int CH = D / 16;                   // 16-byte chunks per row
+    constexpr int SWM = (CH < 8 ? CH : 8) - 1;   // swizzle mask
+    // LDS map (bytes)
+    constexpr int OFF_KS = 0;                    // two fp32 k_scale vectors
+    constexpr int OFF_K = 2 * kBlockN * 4;       // two K tiles
+    constexpr int OFF_V = OFF_K + 2 * KT;        // two V tiles
+    constexpr int LDS_BYTES = OFF_V + 2 * KT;
+    __shared__ __attribute__((aligned(1024))) char smem[LDS_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -48,7 +44,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
     const int n_split = SPLIT ? p.num_splits : 1;
     const int per_head = n_mblk * n_split;
     const int n_heads = p.batch * p.heads;
-    int bid = blockIdx.x;
+    const int bid = blockIdx.x;
     int head, rem;
     if ((n_heads & 7) == 0) {
         const int xcd = bid & 7, slot = bid >> 3;
@@ -70,11 +66,6 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
         const int e = nb_begin + p.blocks_per_split;
         nb_end = e < nb_end ? e : nb_end;
     }
-
-    const char* Kg = p.k + b * p.k_sb + h * p.k_sh;
-    const char* Vg = p.v + b * p.v_sb + h * p.v_sh;
-    const char* Ksg = p.k_scale;
-    const int64_t ks_base = b * p.ks_sb + h * p.ks_sh;
     const int q_row = mb * kBlockM + wave * 32 + lq;     // this lane's query row
 
     // ---- Q fragment (B operand of S^T = K Q^T): 16 bytes per k-step, resident for the whole kernel.
@@ -94,33 +85,45 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
 #pragma unroll
         for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.f;
 
-    // per-lane pieces of the LDS read addresses
-    // K (A operand of S^T): lane reads row (32*st + lq), chunk (2*ks + lh)
-    const int k_swz = swz_k<D>(lq) & ((D / 16 < 8 ? D / 16 : 8) - 1);
-    // V (A operand of O^T = V^T P^T) through the transposing 8-byte load; see intfa_device.h
-    const int g16 = lane >> 4, i16 = lane & 15, jj = i16 >> 1;
-    const int v_row0 = 8 * (jj >> 2) + 4 * lh + (jj & 3);          // + 16*w + 32*st
-    const int v_sub = 8 * (i16 & 1);
-    const int v_swz = swz_v<VROW>(v_row0) & ((VROW / 16 < 8 ? VROW / 16 : 8) - 1);
-
-    const auto k_lane = tile_load_lane<D, false>((uint32_t)p.k_sn, wave, lane);
-    const auto v_lane = tile_load_lane<VROW, true>((uint32_t)p.v_sn, wave, lane);
-    const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen - 1) * p.k_sn + D));
-    const __amdgpu_buffer_rsrc_t v_rsrc = make_rsrc(DUMP_S ? Kg : Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + VROW));
-    auto issue_loads = [&](int nb, char* dK, char* dV) __attribute__((always_inline)) {
-        issue_tile_load<D, false>(k_rsrc, (uint32_t)(nb * kBlockN) * (uint32_t)p.k_sn, (uint32_t)p.k_sn, dK, wave, k_lane);
-        if (!DUMP_S) issue_tile_load<VROW, true>(v_rsrc, (uint32_t)(nb * kBlockN) * (uint32_t)p.v_sn, (uint32_t)p.v_sn, dV, wave, v_lane);
+    // ---- global -> LDS copies (asynchronous, straight into LDS)
+    const char* Kg = p.k + b * p.k_sb + h * p.k_sh;
+    const char* Vg = DUMP_S ? Kg : p.v + b * p.v_sb + h * p.v_sh;
+    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen - 1) * p.k_sn + D));
+    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + D));
+    const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
+    const auto k_lane = tile_load_lane<D, false>(k_sn, wave, lane);
+    const auto v_lane = tile_load_lane<D, true>(v_sn, wave, lane);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    auto issue_loads = [&](int nb, int buf) __attribute__((always_inline)) {
+        issue_tile_load<D, false>(k_rsrc, (uint32_t)(nb * kBlockN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane);
+        if (!DUMP_S) issue_tile_load<D, true>(v_rsrc, (uint32_t)(nb * kBlockN) * v_sn, v_sn, lds0 + OFF_V + buf * KT, wave, v_lane);
     };
-    // k_scale of the block: thread t < 128 fetches the scale of key t, converted to fp32 when stored to LDS
+    // The copy of the NEXT block is issued in slices spread over the stages of the current block (one K slice per
+    // S^T sub-tile stage, one V slice per output d-tile stage) so that the waves do not queue behind a burst.
+    constexpr int DMA_PARTS = TileLoadLane<D, false>::NINST / 4;
+    // When there is no next block the slices are issued against an empty resource (num_records = 0: every access
+    // is out of range and touches no memory), which keeps the stages free of branches.
+    auto issue_k_slice = [&](v4i rsrc, int nb, int buf, int stage, int nstages) __attribute__((always_inline)) {
+#pragma unroll
+        for (int it = 0; it < DMA_PARTS; ++it)
+            if (it * nstages / DMA_PARTS == stage)
+                issue_tile_part<D, false>(rsrc, (uint32_t)(nb * kBlockN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane, it);
+    };
+    auto issue_v_slice = [&](v4i rsrc, int nb, int buf, int stage, int nstages) __attribute__((always_inline)) {
+#pragma unroll
+        for (int it = 0; it < DMA_PARTS; ++it)
+            if (it * nstages / DMA_PARTS == stage)
+                issue_tile_part<D, true>(rsrc, (uint32_t)(nb * kBlockN) * v_sn, v_sn, lds0 + OFF_V + buf * KT, wave, v_lane, it);
+    };
+    // k_scale of a block: thread t < 128 fetches the scale of key t; converted to fp32 when stored to LDS
     const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
-    const __amdgpu_buffer_rsrc_t ks_rsrc =
-        make_rsrc(DUMP_S ? Kg : Ksg + ks_base * ks_esize, DUMP_S ? 0u : (uint32_t)(((p.seqlen - 1) * p.ks_sn + 1) * ks_esize));
-    const uint32_t ks_lane = (uint32_t)(tid & (kBlockN - 1)) * (uint32_t)(p.ks_sn * ks_esize);
-    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {           // raw bits; converted by cvt_ks
+    const char* Ksg = p.k_scale + (b * p.ks_sb + h * p.ks_sh) * ks_esize;
+    const uint32_t ks_goff = (uint32_t)(tid & (kBlockN - 1)) * (uint32_t)(p.ks_sn * ks_esize);
+    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {           // raw bits
         if (DUMP_S) return 0u;
-        const uint32_t so = (uint32_t)(nb * kBlockN) * (uint32_t)(p.ks_sn * ks_esize);
-        if (p.scale_dtype == 2) return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ks_rsrc, ks_lane, so, 0);
-        return (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(ks_rsrc, ks_lane, so, 0);
+        const char* src = Ksg + (int64_t)(nb * kBlockN) * (p.ks_sn * ks_esize);       // wave-uniform part
+        if (p.scale_dtype == 2) return *(const uint32_t*)(src + ks_goff);
+        return (uint32_t)*(const uint16_t*)(src + ks_goff);
     };
     auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float {
         if (p.scale_dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
@@ -128,31 +131,93 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
         return __builtin_bit_cast(float, raw);
     };
 
-    // One key block.  DIAG selects the code for the block on the causal diagonal (mask + sub-tile skip).
-    auto compute = [&](auto diag_tag, int nb, const char* cK, const char* cV, const float* cKs) __attribute__((always_inline)) {
-        constexpr bool DIAG = decltype(diag_tag)::value;
-        // Loop-invariant address pieces are re-derived per block from two opaque values, so the compiler does not
-        // keep a register per (k-step, d-tile) variant alive across the whole loop.
-        int ksw = k_swz, vsw = v_swz;
-        asm volatile("" : "+v"(ksw), "+v"(vsw));
-        // -------- pass 1: S^T sub-tiles, dequantise by k_scale, running row max
-        float t[4][16];
-        float mx = -INFINITY;
+    // ---- per-lane LDS read offsets (everything else is an immediate)
+    // K (A operand of S^T): lane reads row (32*st + lq), chunk (2*ks + lh), XOR-swizzled by the row
+    const int k_swz = swz_k<D>(lq) & SWM;
+    uint32_t k_rd[KS];
 #pragma unroll
-        for (int st = 0; st < 4; ++st) {
+    for (int ks = 0; ks < KS; ++ks) {
+        const int c = 2 * ks + lh;
+        k_rd[ks] = OFF_K + lq * D + (((c & SWM) ^ k_swz) << 4) + ((c & ~SWM) << 4);
+    }
+    // V (A operand of O^T = V^T P^T) through the transposing 8-byte load: source lane s of a 16-lane group points at
+    // key row 8*(j>>2) + 4*lh + (j&3), j = s/2 (+16 for the second load, +32 per sub-tile), 8-byte half s&1
+    const int g16 = lane >> 4, i16 = lane & 15, jj = i16 >> 1;
+    const int v_row0 = 8 * (jj >> 2) + 4 * lh + (jj & 3);
+    const int v_swz = swz_v<D>(v_row0) & SWM;
+    uint32_t v_rd[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const int c = 2 * dt + (g16 & 1);
+        v_rd[dt] = OFF_V + v_row0 * D + 8 * (i16 & 1) + (((c & SWM) ^ v_swz) << 4) + ((c & ~SWM) << 4);
+    }
+    const uint32_t ks_rd = OFF_KS + 16 * lh;     // + 4 * (32*st + 8*a4) per read
+    const uint32_t ks_wr = OFF_KS + 4 * (tid & (kBlockN - 1));
+
+    // One key block out of LDS buffer BUF.  DIAG selects the code for the block on the causal diagonal.
+    auto compute = [&](auto buf_tag, auto diag_tag, int nb, bool more) __attribute__((always_inline)) {
+        constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
+        constexpr bool DIAG = decltype(diag_tag)::value;
+        constexpr int KB = BUF * KT, SB = BUF * kBlockN * 4;
+        v4i k_next = k_rsrc, v_next = v_rsrc;
+        if (!more) { k_next[2] = 0; v_next[2] = 0; }
+        // LDS operand fetches are issued one stage ahead of their MFMAs, in program order pinned by scheduling
+        // barriers: the fragments of sub-tile st+1 (d-tile dt+1) are requested right after the MFMAs of st (dt)
+        // have been issued and arrive while this wave does the vector work of st (dt).
+        auto load_kfrags = [&](v4i (&fr)[KS], int st) __attribute__((always_inline)) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) fr[ks] = *(const v4i*)(smem + k_rd[ks] + KB + 32 * st * D);
+        };
+        auto load_vfrags = [&](v4i (&vf)[NST], int dt) __attribute__((always_inline)) {
+#pragma unroll
+            for (int st = 0; st < NST; ++st) {
+                if (DIAG && st > wave) continue;
+                const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                    (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[dt] + KB + (32 * st) * D));
+                const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                    (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[dt] + KB + (32 * st + 16) * D));
+                vf[st] = (v4i){lo[0], lo[1], hi[0], hi[1]};
+            }
+        };
+        // -------- pass 1: S^T sub-tiles, dequantise by k_scale, running row max.
+        // Software pipeline inside the wave: the MFMA chain of sub-tile st+1 is issued before the vector work of
+        // sub-tile st (the matrix core runs under the wave's own VALU instructions), and LDS operands are requested
+        // two stages before the MFMA that consumes them (double-buffered fragments).
+        const int nact = DIAG ? (wave + 1) : NST;          // active sub-tiles (wave-uniform)
+        float t[NST][16];
+        float mx = -INFINITY;
+        v4i fr[2][KS];
+        v4i vf[2][NST];
+        v16i sacc[2];
+        v4f kk[2][4];
+        auto load_kk = [&](v4f (&dst)[4], int st) __attribute__((always_inline)) {
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4) dst[a4] = *(const v4f*)(smem + ks_rd + SB + 4 * (32 * st + 8 * a4));
+        };
+        auto qk_chain = [&](v16i& acc, const v4i (&f)[KS]) __attribute__((always_inline)) {
+            acc = (v16i){0};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[ks], qreg[ks], acc, 0, 0, 0);
+        };
+        load_kfrags(fr[0], 0);
+        load_kk(kk[0], 0);
+        if (1 < nact) { load_kfrags(fr[1], 1); load_kk(kk[1], 1); }
+        __builtin_amdgcn_sched_barrier(0);
+        qk_chain(sacc[0], fr[0]);
+#pragma unroll
+        for (int st = 0; st < NST; ++st) {
             if (DIAG && st > wave) {                          // sub-tile entirely above the diagonal
 #pragma unroll
                 for (int r = 0; r < 16; ++r) t[st][r] = -INFINITY;
                 continue;
             }
             __builtin_amdgcn_sched_barrier(0);
-            v16i acc = {0};
-            const char* krow = cK + (32 * st + lq) * D;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const v4i a = *(const v4i*)(krow + (((2 * ks + lh) ^ ksw) << 4));
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qreg[ks], acc, 0, 0, 0);
-            }
+            if (st + 1 < NST && st + 1 < nact) qk_chain(sacc[(st + 1) & 1], fr[(st + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (st + 2 < NST && st + 2 < nact) load_kfrags(fr[st & 1], st + 2);
+            if (!DUMP_S && !DIAG) issue_k_slice(k_next, nb + 1, BUF ^ 1, st, NST);
+            __builtin_amdgcn_sched_barrier(0);
+            const v16i& acc = sacc[st & 1];
             if (DUMP_S) {
                 int32_t* srow = p.s_dump + ((int64_t)(b * p.heads + h) * p.seqlen + q_row) * p.seqlen + nb * kBlockN + 32 * st;
 #pragma unroll
@@ -160,10 +225,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
             }
 #pragma unroll
             for (int a4 = 0; a4 < 4; ++a4) {
-                const v4f kk = *(const v4f*)(cKs + 32 * st + 8 * a4 + 4 * lh);
 #pragma unroll
                 for (int b4 = 0; b4 < 4; ++b4) {
-                    float x = (float)acc[4 * a4 + b4] * kk[b4];
+                    float x = (float)acc[4 * a4 + b4] * kk[st & 1][a4][b4];
                     if (DIAG) {
                         // position of the key inside the 32x32 tile on the diagonal vs this lane's query
                         if (st == wave && (8 * a4 + b4) > lq - 4 * lh) x = -INFINITY;
@@ -172,91 +236,103 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
                     mx = fmaxf(mx, x);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
+            if (st + 2 < NST && st + 2 < nact) load_kk(kk[st & 1], st + 2);
         }
         if (DUMP_S) return;
-        mx = fmaxf(mx, wave_half_swap(mx));
+        // V fragments of the first two d-tiles travel while the exponentials are evaluated
+        load_vfrags(vf[0], 0);
+        if (1 < DT) load_vfrags(vf[1], 1);
+        mx = half_pair_max(mx);
         const float m_new = fmaxf(m_run, mx * qsc);
         const float alpha = fast_exp2(m_run - m_new);
         m_run = m_new;
         // -------- pass 2: P = exp2(x*qsc - m), row sum, requantise
         float lsum = 0.f;
-        if (VARIANT == VAR_FULL) {
-            v4i p8[4];
-            const float bias = (PROUND == 0 ? kLog2_127 : 0.f) - m_new;
+        v4i p8[NST];
+        const float bias = (PROUND == 0 ? kLog2_127 : 0.f) - m_new;
 #pragma unroll
-            for (int st = 0; st < 4; ++st) {
-                __builtin_amdgcn_sched_barrier(0);
+        for (int st = 0; st < NST; ++st) {
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int w4 = 0; w4 < 4; ++w4) {
-                    unsigned pk = 0;
-                    if (PROUND == 0) {
+            for (int w4 = 0; w4 < 4; ++w4) {
+                unsigned pk = 0;
+                if (PROUND == 0) {
 #pragma unroll
-                        for (int b4 = 0; b4 < 4; ++b4) {
-                            const float e = fast_exp2(fmaf(t[st][4 * w4 + b4], qsc, bias));   // 127 * p
-                            lsum += e;
-                            pk = __builtin_amdgcn_cvt_pk_u8_f32(e, b4, pk);
-                        }
-                    } else {
-                        // the reference's fp16 chain: fp16(p) * 127 -> fp16, + 0.5 -> fp16, truncate
-#pragma unroll
-                        for (int b4 = 0; b4 < 4; ++b4) {
-                            const float e = fast_exp2(fmaf(t[st][4 * w4 + b4], qsc, bias));   // p
-                            lsum += e;
-                            _Float16 hp = (_Float16)e;
-                            hp = hp * (_Float16)127.0f;
-                            hp = hp + (_Float16)0.5f;
-                            const unsigned q8 = (unsigned)(int)hp;          // truncating convert, 0..127
-                            pk |= q8 << (8 * b4);
-                        }
+                    for (int b4 = 0; b4 < 4; ++b4) {
+                        const float e = fast_exp2(fmaf(t[st][4 * w4 + b4], qsc, bias));   // 127 * p
+                        lsum += e;
+                        pk = __builtin_amdgcn_cvt_pk_u8_f32(e, b4, pk);
                     }
-                    p8[st][w4] = (int)pk;
+                } else {
+                    // the reference's fp16 chain: fp16(p) * 127 -> fp16, + 0.5 -> fp16, truncate
+#pragma unroll
+                    for (int b4 = 0; b4 < 4; ++b4) {
+                        const float e = fast_exp2(fmaf(t[st][4 * w4 + b4], qsc, bias));   // p
+                        lsum += e;
+                        _Float16 hp = (_Float16)e;
+                        hp = hp * (_Float16)127.0f;
+                        hp = hp + (_Float16)0.5f;
+                        const unsigned q8 = (unsigned)(int)hp;          // truncating convert, 0..127
+                        pk |= q8 << (8 * b4);
+                    }
                 }
+                p8[st][w4] = (int)pk;
             }
-            // -------- P V on int8 MFMA: O^T[d, q] += V^T[d, key] P^T[key, q]
-            const char* vbase = cV + v_row0 * VROW + v_sub;
+            asm volatile("" : "+v"(lsum));      // keep the row-sum chain inside its stage
+        }
+        // -------- P V on int8 MFMA: O^T[d, q] += V^T[d, key] P^T[key, q]; the chain of d-tile dt+1 is issued
+        // before the accumulator update of d-tile dt, its V fragments were requested two stages earlier.
+        v16i oacc[2];
+        auto pv_chain = [&](v16i& acc, const v4i (&f)[NST]) __attribute__((always_inline)) {
+            acc = (v16i){0};
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                __builtin_amdgcn_sched_barrier(0);
-                v16i acc = {0};
-                const int coff = ((2 * dt + (g16 & 1)) ^ vsw) << 4;
-#pragma unroll
-                for (int st = 0; st < 4; ++st) {
-                    if (DIAG && st > wave) continue;
-                    const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                        (__attribute__((address_space(3))) v2i*)INTFA_LDS(vbase + (32 * st) * VROW + coff));
-                    const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                        (__attribute__((address_space(3))) v2i*)INTFA_LDS(vbase + (32 * st + 16) * VROW + coff));
-                    const v4i a = {lo[0], lo[1], hi[0], hi[1]};
-                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, p8[st], acc, 0, 0, 0);
-                }
-#pragma unroll
-                for (int r = 0; r < 16; ++r) o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, (float)acc[r]);
+            for (int st = 0; st < NST; ++st) {
+                if (DIAG && st > wave) continue;
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[st], p8[st], acc, 0, 0, 0);
             }
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        pv_chain(oacc[0], vf[0]);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (dt + 1 < DT) pv_chain(oacc[(dt + 1) & 1], vf[(dt + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (dt + 2 < DT) load_vfrags(vf[dt & 1], dt + 2);
+            if (!DIAG) issue_v_slice(v_next, nb + 1, BUF ^ 1, dt, DT);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, (float)oacc[dt & 1][r]);
+
         }
         l_run = fmaf(l_run, alpha, lsum);
     };
+
     // One pipeline step on LDS buffer BUF: wait for this block's tiles (issued one step earlier), make them
     // visible to all four waves, start the copy of the next block into the other buffer, compute.
     auto step = [&](auto buf_tag, auto diag_tag, int nb) __attribute__((always_inline)) {
-        constexpr bool B1 = decltype(buf_tag)::value;
-        char* cK = B1 ? sK1 : sK0; char* cV = B1 ? sV1 : sV0; float* cKs = B1 ? sKs1 : sKs0;
-        char* nK = B1 ? sK0 : sK1; char* nV = B1 ? sV0 : sV1; float* nKs = B1 ? sKs0 : sKs1;
+        constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         const bool more = nb + 1 < nb_end;
         uint32_t ks_next = 0;
-        if (more) { issue_loads(nb + 1, nK, nV); ks_next = load_ks(nb + 1); }
-        compute(diag_tag, nb, cK, cV, cKs);
-        if (more && tid < kBlockN) nKs[tid] = cvt_ks(ks_next);
+        constexpr bool DIAG = decltype(diag_tag)::value;
+        if (more) {
+            if (DUMP_S || DIAG) issue_loads(nb + 1, BUF ^ 1);      // (a diagonal block is the last one: more == false)
+            ks_next = load_ks(nb + 1);
+        }
+        compute(buf_tag, diag_tag, nb, more);
+        if (more && tid < kBlockN) *(float*)(smem + ks_wr + (BUF ^ 1) * kBlockN * 4) = cvt_ks(ks_next);
     };
 
     // ---- main loop: K/V tiles double-buffered in LDS, one barrier per key block.  The block on the causal
     // diagonal is always the last of the range and gets its own code instance after the loop.
     if (nb_begin < nb_end) {
-        issue_loads(nb_begin, sK0, sV0);
+        issue_loads(nb_begin, 0);
         {
             const uint32_t s0 = load_ks(nb_begin);
-            if (tid < kBlockN) sKs0[tid] = cvt_ks(s0);
+            if (tid < kBlockN) *(float*)(smem + ks_wr) = cvt_ks(s0);
         }
         const bool has_diag = CAUSAL && (nb_end == mb + 1);
         const int plain_end = has_diag ? nb_end - 1 : nb_end;
@@ -274,20 +350,20 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
     }
     if (DUMP_S) return;
 
-    // ---- epilogue
-    const float l_tot = l_run + wave_half_swap(l_run);          // in units of 1/127 when PROUND == 0
-    float out_scale;
-    if (VARIANT == VAR_FULL) {
-        const float vs = load_scale(p.v_scale, b * p.vs_sb + h * p.vs_sh, p.scale_dtype);
-        out_scale = (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
-    } else {
-        out_scale = 1.f / l_tot;
-    }
-    const float l_true = (VARIANT == VAR_FULL && PROUND == 0) ? l_tot * (1.f / 127.f) : l_tot;
+    // ---- epilogue.  Everything it needs from the parameter block is (re)loaded here, behind an opaque copy of the
+    // kernel-argument pointer, so that these values do not occupy scalar registers during the main loop.
+    const KParams* pe = (const KParams*)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(pe));
+    const int e_heads = pe->heads, e_seqlen = pe->seqlen;
+    const int eb = head / e_heads, eh = head % e_heads;
+    const float l_tot = half_pair_sum(l_run);          // in units of 1/127 when PROUND == 0
+    const float vs = load_scale(pe->v_scale, eb * pe->vs_sb + eh * pe->vs_sh, pe->scale_dtype);
+    const float out_scale = (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
+    const float l_true = (PROUND == 0) ? l_tot * (1.f / 127.f) : l_tot;
     const float lse = m_run + __builtin_log2f(l_true);
     if (SPLIT) {
-        const int64_t row = ((int64_t)(split * p.batch + b) * p.heads + h) * p.seqlen + q_row;
-        float* op = p.o_part + row * D;
+        const int64_t row = ((int64_t)(split * pe->batch + eb) * e_heads + eh) * e_seqlen + q_row;
+        float* op = pe->o_part + row * D;
         const bool seen = nb_begin < nb_end;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -298,10 +374,10 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
                 for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[dt][4 * a4 + b4] * out_scale : 0.f;
                 *(v4f*)(op + 32 * dt + 8 * a4 + 4 * lh) = o;
             }
-        if (lh == 0) p.lse_part[row] = seen ? lse : -INFINITY;
+        if (lh == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
         return;
     }
-    char* orow = p.out + b * p.o_sb + h * p.o_sh + (int64_t)q_row * p.o_sn;
+    char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -315,16 +391,11 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_int8_kernel(const KParams p) 
             } else {
                 v4s o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) {
-                    const float f = o_acc[dt][4 * a4 + b4] * out_scale;
-                    uint32_t u = __builtin_bit_cast(uint32_t, f);
-                    u += 0x7fffu + ((u >> 16) & 1u);                // round-to-nearest-even to bf16
-                    o[b4] = (short)(u >> 16);
-                }
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(o_acc[dt][4 * a4 + b4] * out_scale);
                 *(v4s*)(orow + d0 * 2) = o;
             }
         }
-    if (p.lse != nullptr && lh == 0) p.lse[((int64_t)(b * p.heads) + h) * p.seqlen + q_row] = lse;
+    if (pe->lse != nullptr && lh == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
 #endif  // __HIP_DEVICE_COMPILE__
 }
 

@@ -38,9 +38,7 @@ __global__ void __launch_bounds__(256) splitkv_combine_kernel(const KParams p) {
         if (OUT_DT == 0) {
             ((_Float16*)orow)[i] = (_Float16)acc[i];
         } else {
-            uint32_t u = __builtin_bit_cast(uint32_t, acc[i]);
-            u += 0x7fffu + ((u >> 16) & 1u);
-            ((uint16_t*)orow)[i] = (uint16_t)(u >> 16);
+            ((uint16_t*)orow)[i] = (uint16_t)f32_to_bf16_bits(acc[i]);
         }
     }
     if (p.lse != nullptr && lane == 0) p.lse[row] = lse;
