@@ -31,6 +31,9 @@ extern "C" {
 
 #define INTFA_VERSION 1
 
+/* forward variants (one entry point each, below) */
+enum { INTFA_VARIANT_FULL_INT8 = 0, INTFA_VARIANT_HALF_INT8 = 1, INTFA_VARIANT_FP16 = 2 };
+
 /* element types of scales / float tensors */
 enum { INTFA_F16 = 0, INTFA_BF16 = 1, INTFA_F32 = 2 };
 
@@ -46,7 +49,7 @@ enum {
     INTFA_OK = 0,
     INTFA_ERR_NULL = -1,          /* a required pointer is NULL */
     INTFA_ERR_HEAD_DIM = -2,      /* head_dim not supported by the kernels */
-    INTFA_ERR_SEQLEN = -3,        /* seqlen not a positive multiple of the key block (128) */
+    INTFA_ERR_SEQLEN = -3,        /* seqlen not a positive multiple of the query block (128) */
     INTFA_ERR_ALIGN = -4,         /* pointer or row stride not 16-byte aligned */
     INTFA_ERR_DTYPE = -5,         /* unknown dtype enum */
     INTFA_ERR_WORKSPACE = -6,     /* workspace missing or too small for the requested split count */
@@ -100,9 +103,10 @@ int intfa_version(void);
 /* Human-readable text for a negative return code; for a positive one returns "hip error". */
 const char* intfa_error_string(int code);
 
-/* Key-block length the kernels quantise P against (the reference's BLOCK_N, an autotuned value there:
- * configs.py:13-19).  A bit-faithful CPU evaluation must use the same value. */
-int intfa_block_n(void);
+/* Key-block length of a variant at a head_dim (the reference's BLOCK_N, an autotuned value there:
+ * configs.py:13-19).  The running max and, on the full-int8 path, the requantisation of P advance per key block,
+ * so a bit-faithful CPU evaluation must use the same value.  Negative INTFA_ERR_* for unknown arguments. */
+int intfa_fwd_block_n(int variant, int head_dim);
 
 /* Bytes of workspace the forward needs for p->num_splits (0 when num_splits <= 1). */
 size_t intfa_fwd_workspace_bytes(const intfa_fwd_params* p);

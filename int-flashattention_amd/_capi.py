@@ -33,7 +33,9 @@ class FwdParams(ctypes.Structure):
     )
 
 
-EXPORTS = ("intfa_version", "intfa_error_string", "intfa_block_n", "intfa_fwd_workspace_bytes",
+VARIANT_FULL_INT8, VARIANT_HALF_INT8, VARIANT_FP16 = 0, 1, 2
+
+EXPORTS = ("intfa_version", "intfa_error_string", "intfa_fwd_block_n", "intfa_fwd_workspace_bytes",
            "intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16", "intfa_debug_qk_int32")
 
 _lib = None
@@ -52,8 +54,8 @@ def load():
     pp = ctypes.POINTER(FwdParams)
     lib.intfa_version.restype = ctypes.c_int
     lib.intfa_version.argtypes = []
-    lib.intfa_block_n.restype = ctypes.c_int
-    lib.intfa_block_n.argtypes = []
+    lib.intfa_fwd_block_n.restype = ctypes.c_int
+    lib.intfa_fwd_block_n.argtypes = [ctypes.c_int, ctypes.c_int]
     lib.intfa_error_string.restype = ctypes.c_char_p
     lib.intfa_error_string.argtypes = [ctypes.c_int]
     lib.intfa_fwd_workspace_bytes.restype = ctypes.c_size_t

@@ -11,7 +11,16 @@ import torch.nn.functional as F
 from . import _capi
 
 _TORCH_TO_ENUM = {torch.float16: _capi.INTFA_F16, torch.bfloat16: _capi.INTFA_BF16, torch.float32: _capi.INTFA_F32}
-BLOCK = 128          # query/key block of the kernels; the sequence length must be a multiple of it
+BLOCK = 128          # query block of the kernels; the sequence length must be a multiple of it
+_VARIANT_ENUM = {"full": _capi.VARIANT_FULL_INT8, "half": _capi.VARIANT_HALF_INT8, "fp": _capi.VARIANT_FP16}
+
+
+def block_n(variant: str, head_dim: int) -> int:
+    """Key-block length the kernel of `variant` ("full", "half", "fp") uses at `head_dim` (the reference's BLOCK_N)."""
+    rc = _capi.load().intfa_fwd_block_n(_VARIANT_ENUM[variant], max(int(head_dim), MIN_HEAD_DIM))
+    if rc < 0:
+        _capi.check(rc, "intfa_fwd_block_n")
+    return rc
 MIN_HEAD_DIM = 64    # smaller head dims are zero-padded up to this (QK^T and the kept output columns are unchanged)
 
 

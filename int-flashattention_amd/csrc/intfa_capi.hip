@@ -1,8 +1,7 @@
 // C ABI of libintfa.so: argument validation, kernel selection and launch.  See include/intfa.h.
 #include "../../include/intfa.h"
 #include "intfa_device.h"
-#include "intfa_fwd_int8.h"
-#include "intfa_fwd_fp16.h"
+#include "intfa_launch.h"
 #include "intfa_splitkv.h"
 
 using namespace intfa;
@@ -19,7 +18,7 @@ int scale_size(int dt) { return dt == INTFA_F32 ? 4 : 2; }
 int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need_scales, bool need_vscale, KParams* kp) {
     if (p == nullptr || p->q == nullptr || p->k == nullptr) return INTFA_ERR_NULL;
     if (p->batch <= 0 || p->heads <= 0) return INTFA_ERR_SHAPE;
-    if (p->seqlen <= 0 || p->seqlen % kBlockN != 0) return INTFA_ERR_SEQLEN;
+    if (p->seqlen <= 0 || p->seqlen % kBlockM != 0) return INTFA_ERR_SEQLEN;
     if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256) return INTFA_ERR_HEAD_DIM;
     if (p->scale_dtype < 0 || p->scale_dtype > 2) return INTFA_ERR_DTYPE;
     if (p->io_dtype != INTFA_F16 && p->io_dtype != INTFA_BF16) return INTFA_ERR_DTYPE;
@@ -55,7 +54,7 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
     k.lse = p->lse;
     k.batch = p->batch; k.heads = p->heads; k.seqlen = p->seqlen; k.head_dim = p->head_dim;
     k.scale_dtype = p->scale_dtype; k.causal = p->causal ? 1 : 0;
-    k.num_splits = 1; k.blocks_per_split = p->seqlen / kBlockN;
+    k.num_splits = 1; k.blocks_per_split = p->seqlen;   // single pass: never the limit
     k.qk_scale_log2 = p->sm_scale * 1.44269504f;      // flash_atten_full_int8.py:156-157
     *kp = k;
     return INTFA_OK;
@@ -67,25 +66,18 @@ size_t workspace_bytes_for(const intfa_fwd_params* p) {
     return rows * (size_t)p->head_dim * sizeof(float) + rows * sizeof(float);
 }
 
-int setup_split(const intfa_fwd_params* p, KParams* kp) {
+int setup_split(const intfa_fwd_params* p, int block_n, KParams* kp) {
     if (p->num_splits <= 1) return INTFA_OK;
     if (p->num_splits > kMaxSplits) return INTFA_ERR_SPLITS;
     const size_t need = workspace_bytes_for(p);
     if (p->workspace == nullptr || p->workspace_bytes < need || !aligned16(p->workspace)) return INTFA_ERR_WORKSPACE;
-    const int n_blocks = p->seqlen / kBlockN;
+    const int n_blocks = p->seqlen / block_n;
     kp->num_splits = p->num_splits;
     kp->blocks_per_split = (n_blocks + p->num_splits - 1) / p->num_splits;     // csrc/flash_fwd_kernel.h:503
     const size_t rows = (size_t)p->num_splits * p->batch * p->heads * p->seqlen;
     kp->o_part = (float*)p->workspace;
     kp->lse_part = kp->o_part + rows * (size_t)p->head_dim;
     return INTFA_OK;
-}
-
-template <typename K> int launch(K kernel, const KParams& kp, hipStream_t stream) {
-    const int grid = kp.batch * kp.heads * (kp.seqlen / kBlockM) * kp.num_splits;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, stream, kp);
-    const hipError_t e = hipGetLastError();
-    return e == hipSuccess ? INTFA_OK : (int)e;
 }
 
 int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t stream) {
@@ -100,25 +92,47 @@ int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t str
     return e == hipSuccess ? INTFA_OK : (int)e;
 }
 
-// Expands the runtime switches (head_dim, causal, out dtype, P rounding, split) into template arguments.
-int dispatch_full_int8(const intfa_fwd_params* p, const KParams& kp, hipStream_t stream) {
-    const bool causal = kp.causal != 0, bf = p->io_dtype == INTFA_BF16, split = kp.num_splits > 1;
-    const int pr = (p->p_round == INTFA_PROUND_REFERENCE) ? 1 : 0;
-#define INTFA_L(DD, C, O, PR, SP) return launch(fwd_full_int8_kernel<DD, C, O, PR, false, SP>, kp, stream)
-#define INTFA_SW_SP(DD, C, O, PR) do { if (split) INTFA_L(DD, C, O, PR, true); else INTFA_L(DD, C, O, PR, false); } while (0)
-#define INTFA_SW_PR(DD, C, O) do { if (pr) INTFA_SW_SP(DD, C, O, 1); else INTFA_SW_SP(DD, C, O, 0); } while (0)
-#define INTFA_SW_O(DD, C) do { if (bf) INTFA_SW_PR(DD, C, 1); else INTFA_SW_PR(DD, C, 0); } while (0)
-#define INTFA_SW_C(DD) do { if (causal) INTFA_SW_O(DD, true); else INTFA_SW_O(DD, false); } while (0)
-    switch (kp.head_dim) {
-        case 64: INTFA_SW_C(64);
-        case 128: INTFA_SW_C(128);
+// Key-block length of a variant at a head_dim: the full-int8 kernel takes 128 keys per block (64 at head_dim 256),
+// the kernels with a 16-bit P V take 64.
+int block_n_for(int variant, int head_dim) {
+    if (variant == INTFA_VARIANT_FULL_INT8) return head_dim <= 128 ? 128 : 64;
+    return 64;
+}
+
+int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dump_s, hipStream_t stream) {
+    LaunchSel sel;
+    sel.causal = kp.causal != 0;
+    sel.io_dt = p->io_dtype == INTFA_BF16 ? 1 : 0;
+    sel.p_round = p->p_round == INTFA_PROUND_REFERENCE ? 1 : 0;
+    sel.split = kp.num_splits > 1;
+    sel.dump_s = dump_s;
+    const int d = kp.head_dim;
+    if (variant == INTFA_VARIANT_FULL_INT8) {
+        if (d == 64) return launch_full_int8_d64(kp, sel, stream);
+        if (d == 128) return launch_full_int8_d128(kp, sel, stream);
+        if (d == 256) return launch_full_int8_d256(kp, sel, stream);
+    } else if (variant == INTFA_VARIANT_HALF_INT8) {
+        if (d == 64) return launch_half_int8_d64(kp, sel, stream);
+        if (d == 128) return launch_half_int8_d128(kp, sel, stream);
+        if (d == 256) return launch_half_int8_d256(kp, sel, stream);
+    } else {
+        if (d == 64) return launch_fp16_d64(kp, sel, stream);
+        if (d == 128) return launch_fp16_d128(kp, sel, stream);
+        if (d == 256) return launch_fp16_d256(kp, sel, stream);
     }
-#undef INTFA_L
-#undef INTFA_SW_SP
-#undef INTFA_SW_PR
-#undef INTFA_SW_O
-#undef INTFA_SW_C
     return INTFA_ERR_HEAD_DIM;
+}
+
+int run_forward(int variant, const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool scales, bool vscale, hipStream_t stream) {
+    KParams kp;
+    int rc = make_kparams(p, qk_bytes, v_bytes, scales, vscale, &kp);
+    if (rc != INTFA_OK) return rc;
+    if (variant == INTFA_VARIANT_FULL_INT8 && p->p_round != INTFA_PROUND_RNE && p->p_round != INTFA_PROUND_REFERENCE) return INTFA_ERR_DTYPE;
+    rc = setup_split(p, block_n_for(variant, kp.head_dim), &kp);
+    if (rc != INTFA_OK) return rc;
+    rc = dispatch(variant, p, kp, false, stream);
+    if (rc != INTFA_OK || kp.num_splits <= 1) return rc;
+    return launch_combine(p, kp, stream);
 }
 
 }  // namespace
@@ -127,7 +141,11 @@ extern "C" {
 
 int intfa_version(void) { return INTFA_VERSION; }
 
-int intfa_block_n(void) { return kBlockN; }
+int intfa_fwd_block_n(int variant, int head_dim) {
+    if (variant < INTFA_VARIANT_FULL_INT8 || variant > INTFA_VARIANT_FP16) return INTFA_ERR_DTYPE;
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256) return INTFA_ERR_HEAD_DIM;
+    return block_n_for(variant, head_dim);
+}
 
 const char* intfa_error_string(int code) {
     switch (code) {
@@ -147,35 +165,15 @@ const char* intfa_error_string(int code) {
 size_t intfa_fwd_workspace_bytes(const intfa_fwd_params* p) { return workspace_bytes_for(p); }
 
 int intfa_fwd_full_int8(const intfa_fwd_params* p, void* stream) {
-    KParams kp;
-    int rc = make_kparams(p, 1, 1, true, true, &kp);
-    if (rc != INTFA_OK) return rc;
-    if (p->p_round != INTFA_PROUND_RNE && p->p_round != INTFA_PROUND_REFERENCE) return INTFA_ERR_DTYPE;
-    rc = setup_split(p, &kp);
-    if (rc != INTFA_OK) return rc;
-    rc = dispatch_full_int8(p, kp, (hipStream_t)stream);
-    if (rc != INTFA_OK || kp.num_splits <= 1) return rc;
-    return launch_combine(p, kp, (hipStream_t)stream);
+    return run_forward(INTFA_VARIANT_FULL_INT8, p, 1, 1, true, true, (hipStream_t)stream);
 }
 
 int intfa_fwd_half_int8(const intfa_fwd_params* p, void* stream) {
-    KParams kp;
-    int rc = make_kparams(p, 1, 2, true, false, &kp);
-    if (rc != INTFA_OK) return rc;
-    rc = setup_split(p, &kp);
-    if (rc != INTFA_OK) return rc;
-    return -100;
+    return run_forward(INTFA_VARIANT_HALF_INT8, p, 1, 2, true, false, (hipStream_t)stream);
 }
 
 int intfa_fwd_fp16(const intfa_fwd_params* p, void* stream) {
-    KParams kp;
-    int rc = make_kparams(p, 2, 2, false, false, &kp);
-    if (rc != INTFA_OK) return rc;
-    rc = setup_split(p, &kp);
-    if (rc != INTFA_OK) return rc;
-    rc = dispatch_fp16(p, kp, (hipStream_t)stream);
-    if (rc != INTFA_OK || kp.num_splits <= 1) return rc;
-    return launch_combine(p, kp, (hipStream_t)stream);
+    return run_forward(INTFA_VARIANT_FP16, p, 2, 2, false, false, (hipStream_t)stream);
 }
 
 int intfa_debug_qk_int32(const intfa_fwd_params* p, int32_t* s_out, void* stream) {
@@ -186,11 +184,7 @@ int intfa_debug_qk_int32(const intfa_fwd_params* p, int32_t* s_out, void* stream
     kp.s_dump = s_out;
     kp.causal = 0;
     kp.scale_dtype = INTFA_F32;
-    switch (kp.head_dim) {
-        case 64: return launch(fwd_full_int8_kernel<64, false, 0, 0, true, false>, kp, (hipStream_t)stream);
-        case 128: return launch(fwd_full_int8_kernel<128, false, 0, 0, true, false>, kp, (hipStream_t)stream);
-    }
-    return INTFA_ERR_HEAD_DIM;
+    return dispatch(INTFA_VARIANT_FULL_INT8, p, kp, true, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -35,7 +35,7 @@ typedef short v4s __attribute__((ext_vector_type(4)));
 #define INTFA_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
 
 constexpr int kBlockM = 128;
-constexpr int kBlockN = 128;
+constexpr int kBlockN = 128;                  // key block of the full-int8 kernel for head_dim <= 128
 constexpr int kThreads = 256;
 constexpr float kLog2_127 = 6.98868468677f;   // log2(127)
 
@@ -64,43 +64,54 @@ __device__ __forceinline__ float load_scale(const char* base, int64_t idx, int d
     return ((const float*)base)[idx];
 }
 
-// ---- LDS swizzles.  A tile row is D bytes; its 16-byte chunks are XOR-permuted with a function of the row so
-// that the 8 rows touched together by one group of lanes fall into 8 different bank groups.
-// K rows are read by 8 consecutive lanes as 8 consecutive rows.
+// ---- LDS swizzles.  A tile row is ROW_BYTES bytes; its 16-byte chunks are XOR-permuted with a function of the
+// row so that the rows touched together by one LDS access cycle (64 banks x 4 bytes = 256 bytes: 16 lanes of a
+// 16-byte read, 32 lanes of an 8-byte read) fall into different bank groups.  Every function depends on the low
+// four bits of the row only.
+enum { SWZ_K = 0, SWZ_V8 = 1, SWZ_V16 = 2 };
+// K / Q style rows: 16 consecutive lanes read the same chunk of 16 consecutive rows.
 template <int ROW_BYTES> __device__ __forceinline__ int swz_k(int row) {
-    if (ROW_BYTES >= 128) return (row & 7) ^ ((row >> 3) & 1);   // 16 consecutive rows -> 16 distinct 16-byte bank groups
-    return (row >> 1) & 3;                       // 64-byte rows: two rows share a 128-byte line
+    if (ROW_BYTES >= 256) return row & 15;                           // every row starts at bank 0
+    if (ROW_BYTES == 128) return (row & 7) ^ ((row >> 3) & 1);       // rows r, r+8 share banks: flip bit 0
+    return (row >> 1) & 3;                                           // 64-byte rows: 4 rows per 256 bytes
 }
-// V rows are read by the transposing load as rows {0,1,2,3,8,9,10,11} + 4h of a 32-key sub-tile.
-template <int ROW_BYTES> __device__ __forceinline__ int swz_v(int row) {
+// int8 V rows read by ds_read_b64_tr_b8: a 16-lane group touches rows {0,1,2,3,8,9,10,11} + 4h of a sub-tile.
+template <int ROW_BYTES> __device__ __forceinline__ int swz_v8(int row) {
     if (ROW_BYTES >= 128) return (row & 3) | ((row >> 1) & 4);
     return ((row >> 1) & 1) | ((row >> 2) & 2);
 }
+// 16-bit V rows read by ds_read_b64_tr_b16: 32 lanes touch 4 consecutive rows x 64 contiguous bytes.
+template <int ROW_BYTES> __device__ __forceinline__ int swz_v16(int row) {
+    if (ROW_BYTES >= 256) return (row & 3) << 2;
+    return ((row >> 1) & 1) << 2;                                    // 128-byte rows: rows r, r+1 differ by half
+}
+template <int ROW_BYTES, int SWZ> __device__ __forceinline__ int swz(int row) {
+    return SWZ == SWZ_K ? swz_k<ROW_BYTES>(row) : (SWZ == SWZ_V8 ? swz_v8<ROW_BYTES>(row) : swz_v16<ROW_BYTES>(row));
+}
 
-// Asynchronous copy of one 128-row tile (ROW_BYTES bytes per row) from global memory straight into LDS with
-// global_load_lds_dwordx4: every wave instruction moves 64 x 16 bytes into 1 KiB of consecutive LDS, so the
+// Asynchronous copy of one ROWS-row tile (ROW_BYTES bytes per row) from global memory straight into LDS with
+// buffer_load_dwordx4 ... lds: every wave instruction moves 64 x 16 bytes into 1 KiB of consecutive LDS, so the
 // swizzle is applied on the GLOBAL side (which chunk a lane fetches).  The four waves split the instructions.
-// Addressing is split into a wave-uniform 64-bit base (SGPRs) and a per-lane 32-bit offset.  The swizzle of a
-// row depends on the row's low four bits only; wave w issues instructions w, w+4, w+8, ... whose first rows
-// differ by multiples of 4*RPI rows, so a lane needs one offset when 4*RPI >= 16 and two otherwise.
-template <int ROW_BYTES, bool IS_V> struct TileLoadLane {
+// Addressing is split into a wave-uniform part (SGPRs) and a per-lane 32-bit offset.  The swizzle of a row depends
+// on the row's low four bits only; wave w issues instructions w, w+4, w+8, ... whose first rows differ by
+// multiples of 4*RPI rows, so a lane needs one offset when 4*RPI >= 16 and 16/(4*RPI) otherwise.
+template <int ROW_BYTES, int SWZ, int ROWS> struct TileLoadLane {
     static constexpr int CH = ROW_BYTES / 16;        // 16-byte chunks per row
     static constexpr int RPI = 64 / CH;              // rows per wave instruction
-    static constexpr int NINST = kBlockN * CH / 64;  // wave instructions per tile
+    static constexpr int NINST = ROWS * CH / 64;     // wave instructions per tile
     static constexpr int NV = (4 * RPI >= 16) ? 1 : 16 / (4 * RPI);
-    static_assert(RPI >= 2 && RPI <= 16 && NINST % 4 == 0, "unsupported row size");
+    static_assert(CH >= 4 && CH <= 32 && NINST % 4 == 0, "unsupported tile geometry");
     uint32_t off[NV];
 };
-template <int ROW_BYTES, bool IS_V>
-__device__ __forceinline__ TileLoadLane<ROW_BYTES, IS_V> tile_load_lane(uint32_t row_stride, int wave, int lane) {
-    using T = TileLoadLane<ROW_BYTES, IS_V>;
-    constexpr int SM = (T::CH < 8 ? T::CH : 8) - 1;
+template <int ROW_BYTES, int SWZ, int ROWS>
+__device__ __forceinline__ TileLoadLane<ROW_BYTES, SWZ, ROWS> tile_load_lane(uint32_t row_stride, int wave, int lane) {
+    using T = TileLoadLane<ROW_BYTES, SWZ, ROWS>;
     const int rsub = lane / T::CH, cp = lane % T::CH;
     T t;
 #pragma unroll
     for (int v = 0; v < T::NV; ++v) {
         const int row = (v * 4 + wave) * T::RPI + rsub;
-        const int f = (IS_V ? swz_v<ROW_BYTES>(row) : swz_k<ROW_BYTES>(row)) & SM;
+        const int f = swz<ROW_BYTES, SWZ>(row) & (T::CH - 1);
         t.off[v] = (uint32_t)rsub * row_stride + (uint32_t)((cp ^ f) << 4);
     }
     return t;
@@ -120,22 +131,22 @@ __device__ __forceinline__ v4i make_rsrc(const void* base, uint32_t bytes) {
     return r;
 }
 // Issues wave instruction number `it` (0 .. NINST/4 - 1) of this wave's share of one tile copy.
-template <int ROW_BYTES, bool IS_V>
+template <int ROW_BYTES, int SWZ, int ROWS>
 __device__ __forceinline__ void issue_tile_part(v4i rsrc, uint32_t tile_off, uint32_t row_stride, uint32_t lds_tile,
-                                                int wave, const TileLoadLane<ROW_BYTES, IS_V>& ln, int it) {
-    using T = TileLoadLane<ROW_BYTES, IS_V>;
+                                                int wave, const TileLoadLane<ROW_BYTES, SWZ, ROWS>& ln, int it) {
+    using T = TileLoadLane<ROW_BYTES, SWZ, ROWS>;
     const int i = it * 4 + wave;                     // wave-uniform instruction index
     const uint32_t m0v = lds_tile + (uint32_t)i * 1024u;
     const uint32_t soff = tile_off + (uint32_t)(i * T::RPI) * row_stride;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :: "s"(m0v), "v"(ln.off[it % T::NV]), "s"(rsrc), "s"(soff) : "memory");
 }
-template <int ROW_BYTES, bool IS_V>
+template <int ROW_BYTES, int SWZ, int ROWS>
 __device__ __forceinline__ void issue_tile_load(v4i rsrc, uint32_t tile_off, uint32_t row_stride, uint32_t lds_tile,
-                                                int wave, const TileLoadLane<ROW_BYTES, IS_V>& ln) {
-    using T = TileLoadLane<ROW_BYTES, IS_V>;
+                                                int wave, const TileLoadLane<ROW_BYTES, SWZ, ROWS>& ln) {
+    using T = TileLoadLane<ROW_BYTES, SWZ, ROWS>;
 #pragma unroll
-    for (int it = 0; it < T::NINST / 4; ++it) issue_tile_part<ROW_BYTES, IS_V>(rsrc, tile_off, row_stride, lds_tile, wave, ln, it);
+    for (int it = 0; it < T::NINST / 4; ++it) issue_tile_part<ROW_BYTES, SWZ, ROWS>(rsrc, tile_off, row_stride, lds_tile, wave, ln, it);
 }
 
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {   // round-to-nearest-even

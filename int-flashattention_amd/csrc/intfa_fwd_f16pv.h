@@ -1,0 +1,315 @@
+// Forward kernel with P V on 16-bit floating-point MFMA: the half-int8 variant (int8 Q K^T with per-token
+// scales, flash_atten_int8.py:9-66) and the fp16/bf16 variant (flash_atten_fp.py:9-60).
+//
+// Same tiling as the full-int8 kernel (4 waves x 32 query rows, S^T = K Q^T so that a lane owns one query
+// column), but keys go in blocks of 64 (two 32-key sub-tiles) and P is cast to V's 16-bit type in registers
+// and multiplied on v_mfma_f32_32x32x16_{f16,bf16}, whose fp32 accumulator IS the running output: per block the
+// accumulator is scaled by alpha and the MFMA adds P V on top (acc = tl.dot(p, v, acc), flash_atten_int8.py:59).
+// V rows stay row-major in LDS; the transposing 8-byte load (ds_read_b64_tr_b16) delivers the A operand.
+#pragma once
+#include "intfa_device.h"
+#include "intfa_fwd_int8.h"
+
+namespace intfa {
+
+constexpr int kBlockN16 = 64;      // key block of this kernel
+
+__device__ __forceinline__ v8h pack_p_f16(const float* e) {
+    v8h r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = (_Float16)e[i];
+    return r;
+}
+__device__ __forceinline__ v8bf pack_p_bf16(const float* e) {
+    v8bf r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = __builtin_bit_cast(__bf16, (uint16_t)f32_to_bf16_bits(e[i]));
+    return r;
+}
+
+// QK_INT8: int8 Q/K with scales (half-int8) or 16-bit Q/K (fp16/bf16 variant).  IO_DT: type of V, P and the output
+// (and of Q/K when !QK_INT8): 0 fp16, 1 bf16.
+template <bool QK_INT8, int D, bool CAUSAL, int IO_DT, bool SPLIT>
+__global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel(const KParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int BN = kBlockN16, NST = BN / 32;
+    constexpr int RDIAG = kBlockM / BN;               // key blocks overlapping the diagonal of a query block
+    constexpr int QB = QK_INT8 ? 1 : 2;               // bytes per Q/K element
+    constexpr int KROW = D * QB, VROW = D * 2;        // bytes per K / V row
+    constexpr int KS = KROW / 32;                     // MFMA k-steps of S^T (32 bytes of a row each)
+    constexpr int DT = D / 32;                        // 32-wide output tiles
+    constexpr int KT = BN * KROW, VT = BN * VROW;
+    constexpr int KCH = KROW / 16, VCH = VROW / 16;
+    constexpr int OFF_KS = 0;
+    constexpr int OFF_K = 2 * BN * 4;
+    constexpr int OFF_V = OFF_K + 2 * KT;
+    constexpr int LDS_BYTES = OFF_V + 2 * VT;
+    __shared__ __attribute__((aligned(1024))) char smem[LDS_BYTES];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lq = lane & 31, lh = lane >> 5;
+
+    const int n_mblk = p.seqlen / kBlockM;
+    const int n_split = SPLIT ? p.num_splits : 1;
+    const int per_head = n_mblk * n_split;
+    const int n_heads = p.batch * p.heads;
+    const int bid = blockIdx.x;
+    int head, rem;
+    if ((n_heads & 7) == 0) {                         // whole heads per XCD (see the full-int8 kernel)
+        const int xcd = bid & 7, slot = bid >> 3;
+        head = (slot / per_head) * 8 + xcd;
+        rem = slot % per_head;
+    } else {
+        head = bid / per_head;
+        rem = bid % per_head;
+    }
+    int mb = rem / n_split;
+    const int split = rem % n_split;
+    if (CAUSAL) mb = n_mblk - 1 - mb;
+    const int b = head / p.heads, h = head % p.heads;
+    int nb_begin = 0, nb_end = CAUSAL ? (mb + 1) * RDIAG : (p.seqlen / BN);
+    if (SPLIT) {
+        nb_begin = split * p.blocks_per_split;
+        const int e = nb_begin + p.blocks_per_split;
+        nb_end = e < nb_end ? e : nb_end;
+    }
+    const int q_row = mb * kBlockM + wave * 32 + lq;
+
+    // ---- Q fragments (B operand of S^T): 16 bytes per k-step
+    v4i qreg[KS];
+    {
+        const char* qrow = p.q + b * p.q_sb + h * p.q_sh + (int64_t)q_row * p.q_sn;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qreg[ks] = *(const v4i*)(qrow + ks * 32 + lh * 16);
+    }
+    // exponent scale of this lane's row: q_scale * sm_scale * log2(e) (int8 Q K^T) or sm_scale * log2(e)
+    const float qsc = QK_INT8 ? load_scale(p.q_scale, b * p.qs_sb + h * p.qs_sh + (int64_t)q_row * p.qs_sn, p.scale_dtype) * p.qk_scale_log2
+                              : p.qk_scale_log2;
+    float m_run = -INFINITY, l_run = 0.f;
+    v16f o_acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.f;
+
+    // ---- global -> LDS copies
+    const char* Kg = p.k + b * p.k_sb + h * p.k_sh;
+    const char* Vg = p.v + b * p.v_sb + h * p.v_sh;
+    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen - 1) * p.k_sn + KROW));
+    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + VROW));
+    const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
+    const auto k_lane = tile_load_lane<KROW, SWZ_K, BN>(k_sn, wave, lane);
+    const auto v_lane = tile_load_lane<VROW, SWZ_V16, BN>(v_sn, wave, lane);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    auto issue_loads = [&](int nb, int buf) __attribute__((always_inline)) {
+        issue_tile_load<KROW, SWZ_K, BN>(k_rsrc, (uint32_t)(nb * BN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane);
+        issue_tile_load<VROW, SWZ_V16, BN>(v_rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane);
+    };
+    const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
+    const char* Ksg = QK_INT8 ? p.k_scale + (b * p.ks_sb + h * p.ks_sh) * ks_esize : nullptr;
+    const uint32_t ks_goff = (uint32_t)(tid & (BN - 1)) * (uint32_t)(p.ks_sn * ks_esize);
+    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
+        if (!QK_INT8 || tid >= BN) return 0u;
+        const char* src = Ksg + (int64_t)(nb * BN) * (p.ks_sn * ks_esize);
+        if (p.scale_dtype == 2) return *(const uint32_t*)(src + ks_goff);
+        return (uint32_t)*(const uint16_t*)(src + ks_goff);
+    };
+    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float {
+        if (p.scale_dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+        if (p.scale_dtype == 1) return __builtin_bit_cast(float, raw << 16);
+        return __builtin_bit_cast(float, raw);
+    };
+
+    // ---- per-lane LDS read offsets
+    const int k_swz = swz_k<KROW>(lq) & (KCH - 1);
+    uint32_t k_rd[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) k_rd[ks] = OFF_K + lq * KROW + (((2 * ks + lh) ^ k_swz) << 4);
+    // V through ds_read_b64_tr_b16: inside a 16-lane group, result lane i element j comes from element i%4 of the
+    // 8 bytes addressed by lane 4j + i/4.  Source lane s therefore points at key row (s >> 2) of a run of four
+    // consecutive keys and at the four head-dim values d0 + 4*(s & 3) .. +3, d0 = 32*dt + 16*(group & 1).
+    const int g16 = lane >> 4, s16 = lane & 15;
+    const int v_row0 = 4 * lh + (s16 >> 2);           // + 8*w + 16*u + 32*st
+    const int v_swz = swz_v16<VROW>(v_row0) & (VCH - 1);
+    uint32_t v_rd[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const int c = 4 * dt + 2 * (g16 & 1) + ((s16 & 3) >> 1);
+        v_rd[dt] = OFF_V + v_row0 * VROW + ((c ^ v_swz) << 4) + 8 * (s16 & 1);
+    }
+    const uint32_t ks_rd = OFF_KS + 16 * lh;
+    const uint32_t ks_wr = OFF_KS + 4 * (tid & (BN - 1));
+
+    auto compute = [&](auto buf_tag, auto diag_tag, int nb, int kb) __attribute__((always_inline)) {
+        constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
+        constexpr bool DIAG = decltype(diag_tag)::value;
+        constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4;
+        const int gw = wave - kb * NST;                 // sub-tile on this wave's diagonal (DIAG only)
+        if (DIAG && gw < 0) return;                     // block entirely above the wave's rows
+        // -------- S^T sub-tiles and running max
+        float t[NST][16];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int st = 0; st < NST; ++st) {
+            if (DIAG && st > gw) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) t[st][r] = -INFINITY;
+                continue;
+            }
+            v4i fr[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) fr[ks] = *(const v4i*)(smem + k_rd[ks] + KB + 32 * st * KROW);
+            float x[16];
+            if (QK_INT8) {
+                v16i acc = {0};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[ks], qreg[ks], acc, 0, 0, 0);
+#pragma unroll
+                for (int a4 = 0; a4 < 4; ++a4) {
+                    const v4f kk = *(const v4f*)(smem + ks_rd + SB + 4 * (32 * st + 8 * a4));
+#pragma unroll
+                    for (int b4 = 0; b4 < 4; ++b4) x[4 * a4 + b4] = (float)acc[4 * a4 + b4] * kk[b4];
+                }
+            } else {
+                v16f acc = {0};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    if (IO_DT == 0) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, fr[ks]), __builtin_bit_cast(v8h, qreg[ks]), acc, 0, 0, 0);
+                    else acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fr[ks]), __builtin_bit_cast(v8bf, qreg[ks]), acc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x[r] = acc[r];
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = x[r];
+                if (DIAG && st == gw && (8 * (r >> 2) + (r & 3)) > lq - 4 * lh) v = -INFINITY;
+                t[st][r] = v;
+                mx = fmaxf(mx, v);
+            }
+        }
+        mx = half_pair_max(mx);
+        const float m_new = fmaxf(m_run, mx * qsc);
+        const float alpha = fast_exp2(m_run - m_new);
+        m_run = m_new;
+        // -------- P = exp2(x*qsc - m), row sum, cast to the 16-bit type; rescale the running output
+        float lsum = 0.f;
+        v4i pf[NST][2];                                   // B operands: 8 x 16-bit per 16-key step
+#pragma unroll
+        for (int st = 0; st < NST; ++st) {
+            float e[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { e[r] = fast_exp2(fmaf(t[st][r], qsc, -m_new)); lsum += e[r]; }
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                pf[st][u] = IO_DT == 0 ? __builtin_bit_cast(v4i, pack_p_f16(e + 8 * u)) : __builtin_bit_cast(v4i, pack_p_bf16(e + 8 * u));
+        }
+        l_run = fmaf(l_run, alpha, lsum);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+        // -------- O^T[d, q] += V^T[d, key] P^T[key, q]
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+            for (int st = 0; st < NST; ++st) {
+                if (DIAG && st > gw) continue;
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const uint32_t a0 = v_rd[dt] + VB + (32 * st + 16 * u) * VROW;
+                    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)INTFA_LDS(smem + a0));
+                    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)INTFA_LDS(smem + a0 + 8 * VROW));
+                    const v4i a = {__builtin_bit_cast(v2i, lo)[0], __builtin_bit_cast(v2i, lo)[1], __builtin_bit_cast(v2i, hi)[0], __builtin_bit_cast(v2i, hi)[1]};
+                    if (IO_DT == 0) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, pf[st][u]), o_acc[dt], 0, 0, 0);
+                    else o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, pf[st][u]), o_acc[dt], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    auto step = [&](auto buf_tag, auto diag_tag, int nb) __attribute__((always_inline)) {
+        constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const bool more = nb + 1 < nb_end;
+        uint32_t ks_next = 0;
+        if (more) { issue_loads(nb + 1, BUF ^ 1); ks_next = load_ks(nb + 1); }
+        compute(buf_tag, diag_tag, nb, CAUSAL ? nb - mb * RDIAG : 0);
+        if (QK_INT8 && more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
+    };
+
+    if (nb_begin < nb_end) {
+        issue_loads(nb_begin, 0);
+        if (QK_INT8) {
+            const uint32_t s0 = load_ks(nb_begin);
+            if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
+        }
+        const int diag_begin = mb * RDIAG;
+        const int plain_end = (CAUSAL && nb_end > diag_begin) ? diag_begin : nb_end;
+        int nb = nb_begin;
+        while (true) {
+            if (nb >= plain_end) break;
+            step(BoolTag<false>{}, BoolTag<false>{}, nb++);
+            if (nb >= plain_end) break;
+            step(BoolTag<true>{}, BoolTag<false>{}, nb++);
+        }
+        if (CAUSAL) {
+#pragma unroll
+            for (int kb = 0; kb < RDIAG; ++kb) {
+                if (nb >= nb_end) break;
+                if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb);
+                else step(BoolTag<true>{}, BoolTag<true>{}, nb);
+                ++nb;
+            }
+        }
+    }
+
+    // ---- epilogue
+    const KParams* pe = (const KParams*)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(pe));
+    const int e_heads = pe->heads, e_seqlen = pe->seqlen;
+    const int eb = head / e_heads, eh = head % e_heads;
+    const float l_tot = half_pair_sum(l_run);
+    const float inv = 1.f / l_tot;
+    const float lse = m_run + __builtin_log2f(l_tot);
+    if (SPLIT) {
+        const int64_t row = ((int64_t)(split * pe->batch + eb) * e_heads + eh) * e_seqlen + q_row;
+        float* op = pe->o_part + row * D;
+        const bool seen = nb_begin < nb_end;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4) {
+                v4f o;
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[dt][4 * a4 + b4] * inv : 0.f;
+                *(v4f*)(op + 32 * dt + 8 * a4 + 4 * lh) = o;
+            }
+        if (lh == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
+        return;
+    }
+    char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+            const int d0 = 32 * dt + 8 * a4 + 4 * lh;
+            if (IO_DT == 0) {
+                v4h o;
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(o_acc[dt][4 * a4 + b4] * inv);
+                *(v4h*)(orow + d0 * 2) = o;
+            } else {
+                v4s o;
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(o_acc[dt][4 * a4 + b4] * inv);
+                *(v4s*)(orow + d0 * 2) = o;
+            }
+        }
+    if (pe->lse != nullptr && lh == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
+#endif  // __HIP_DEVICE_COMPILE__
+}
+
+}  // namespace intfa

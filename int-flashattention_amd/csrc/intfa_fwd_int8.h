@@ -18,18 +18,23 @@ namespace intfa {
 
 template <bool V> struct BoolTag { static constexpr bool value = V; };
 
+// Key block length of the full-int8 kernel: 128 keys, or 64 at head_dim 256 (registers and LDS).
+template <int D> struct FullInt8Geom { static constexpr int NST = D <= 128 ? 4 : 2; static constexpr int BN = 32 * NST; };
+
 template <int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUMP_S, bool SPLIT>
-__global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParams p) {
+__global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T (32 bytes of head_dim each)
     constexpr int DT = D / 32;                   // 32-wide output tiles along head_dim
-    constexpr int NST = kBlockN / 32;            // 32-key sub-tiles per key block
-    constexpr int KT = kBlockN * D;              // bytes of one K tile (and of one int8 V tile)
+    constexpr int NST = FullInt8Geom<D>::NST;    // 32-key sub-tiles per key block
+    constexpr int BN = FullInt8Geom<D>::BN;      // keys per block
+    constexpr int RDIAG = kBlockM / BN;          // key blocks that overlap the causal diagonal of a query block
+    constexpr int KT = BN * D;                   // bytes of one K tile (and of one int8 V tile)
     constexpr int CH = D / 16;                   // 16-byte chunks per row
     constexpr int SWM = (CH < 8 ? CH : 8) - 1;   // swizzle mask
     // LDS map (bytes)
     constexpr int OFF_KS = 0;                    // two fp32 k_scale vectors
-    constexpr int OFF_K = 2 * kBlockN * 4;       // two K tiles
+    constexpr int OFF_K = 2 * BN * 4;            // two K tiles
     constexpr int OFF_V = OFF_K + 2 * KT;        // two V tiles
     constexpr int LDS_BYTES = OFF_V + 2 * KT;
     __shared__ __attribute__((aligned(1024))) char smem[LDS_BYTES];
@@ -60,7 +65,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     const int b = head / p.heads, h = head % p.heads;
 
     // key-block range of this workgroup
-    int nb_begin = 0, nb_end = CAUSAL ? (mb + 1) : (p.seqlen / kBlockN);
+    int nb_begin = 0, nb_end = CAUSAL ? (mb + 1) * RDIAG : (p.seqlen / BN);
     if (SPLIT) {
         nb_begin = split * p.blocks_per_split;
         const int e = nb_begin + p.blocks_per_split;
@@ -91,37 +96,37 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen - 1) * p.k_sn + D));
     const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + D));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
-    const auto k_lane = tile_load_lane<D, false>(k_sn, wave, lane);
-    const auto v_lane = tile_load_lane<D, true>(v_sn, wave, lane);
+    const auto k_lane = tile_load_lane<D, SWZ_K, BN>(k_sn, wave, lane);
+    const auto v_lane = tile_load_lane<D, SWZ_V8, BN>(v_sn, wave, lane);
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
     auto issue_loads = [&](int nb, int buf) __attribute__((always_inline)) {
-        issue_tile_load<D, false>(k_rsrc, (uint32_t)(nb * kBlockN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane);
-        if (!DUMP_S) issue_tile_load<D, true>(v_rsrc, (uint32_t)(nb * kBlockN) * v_sn, v_sn, lds0 + OFF_V + buf * KT, wave, v_lane);
+        issue_tile_load<D, SWZ_K, BN>(k_rsrc, (uint32_t)(nb * BN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane);
+        if (!DUMP_S) issue_tile_load<D, SWZ_V8, BN>(v_rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * KT, wave, v_lane);
     };
     // The copy of the NEXT block is issued in slices spread over the stages of the current block (one K slice per
     // S^T sub-tile stage, one V slice per output d-tile stage) so that the waves do not queue behind a burst.
-    constexpr int DMA_PARTS = TileLoadLane<D, false>::NINST / 4;
+    constexpr int DMA_PARTS = TileLoadLane<D, SWZ_K, BN>::NINST / 4;
     // When there is no next block the slices are issued against an empty resource (num_records = 0: every access
     // is out of range and touches no memory), which keeps the stages free of branches.
     auto issue_k_slice = [&](v4i rsrc, int nb, int buf, int stage, int nstages) __attribute__((always_inline)) {
 #pragma unroll
         for (int it = 0; it < DMA_PARTS; ++it)
             if (it * nstages / DMA_PARTS == stage)
-                issue_tile_part<D, false>(rsrc, (uint32_t)(nb * kBlockN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane, it);
+                issue_tile_part<D, SWZ_K, BN>(rsrc, (uint32_t)(nb * BN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane, it);
     };
     auto issue_v_slice = [&](v4i rsrc, int nb, int buf, int stage, int nstages) __attribute__((always_inline)) {
 #pragma unroll
         for (int it = 0; it < DMA_PARTS; ++it)
             if (it * nstages / DMA_PARTS == stage)
-                issue_tile_part<D, true>(rsrc, (uint32_t)(nb * kBlockN) * v_sn, v_sn, lds0 + OFF_V + buf * KT, wave, v_lane, it);
+                issue_tile_part<D, SWZ_V8, BN>(rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * KT, wave, v_lane, it);
     };
     // k_scale of a block: thread t < 128 fetches the scale of key t; converted to fp32 when stored to LDS
     const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
     const char* Ksg = p.k_scale + (b * p.ks_sb + h * p.ks_sh) * ks_esize;
-    const uint32_t ks_goff = (uint32_t)(tid & (kBlockN - 1)) * (uint32_t)(p.ks_sn * ks_esize);
+    const uint32_t ks_goff = (uint32_t)(tid & (BN - 1)) * (uint32_t)(p.ks_sn * ks_esize);
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {           // raw bits
         if (DUMP_S) return 0u;
-        const char* src = Ksg + (int64_t)(nb * kBlockN) * (p.ks_sn * ks_esize);       // wave-uniform part
+        const char* src = Ksg + (int64_t)(nb * BN) * (p.ks_sn * ks_esize);       // wave-uniform part
         if (p.scale_dtype == 2) return *(const uint32_t*)(src + ks_goff);
         return (uint32_t)*(const uint16_t*)(src + ks_goff);
     };
@@ -133,18 +138,17 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
 
     // ---- per-lane LDS read offsets (everything else is an immediate)
     // K (A operand of S^T): lane reads row (32*st + lq), chunk (2*ks + lh), XOR-swizzled by the row
-    const int k_swz = swz_k<D>(lq) & SWM;
+    const int k_swz = swz_k<D>(lq) & (CH - 1);
     uint32_t k_rd[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        const int c = 2 * ks + lh;
-        k_rd[ks] = OFF_K + lq * D + (((c & SWM) ^ k_swz) << 4) + ((c & ~SWM) << 4);
+        k_rd[ks] = OFF_K + lq * D + (((2 * ks + lh) ^ k_swz) << 4);
     }
     // V (A operand of O^T = V^T P^T) through the transposing 8-byte load: source lane s of a 16-lane group points at
     // key row 8*(j>>2) + 4*lh + (j&3), j = s/2 (+16 for the second load, +32 per sub-tile), 8-byte half s&1
     const int g16 = lane >> 4, i16 = lane & 15, jj = i16 >> 1;
     const int v_row0 = 8 * (jj >> 2) + 4 * lh + (jj & 3);
-    const int v_swz = swz_v<D>(v_row0) & SWM;
+    const int v_swz = swz_v8<D>(v_row0) & SWM;
     uint32_t v_rd[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
@@ -152,13 +156,18 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         v_rd[dt] = OFF_V + v_row0 * D + 8 * (i16 & 1) + (((c & SWM) ^ v_swz) << 4) + ((c & ~SWM) << 4);
     }
     const uint32_t ks_rd = OFF_KS + 16 * lh;     // + 4 * (32*st + 8*a4) per read
-    const uint32_t ks_wr = OFF_KS + 4 * (tid & (kBlockN - 1));
+    const uint32_t ks_wr = OFF_KS + 4 * (tid & (BN - 1));
 
     // One key block out of LDS buffer BUF.  DIAG selects the code for the block on the causal diagonal.
-    auto compute = [&](auto buf_tag, auto diag_tag, int nb, bool more) __attribute__((always_inline)) {
+    auto compute = [&](auto buf_tag, auto diag_tag, int nb, bool more, int kb) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         constexpr bool DIAG = decltype(diag_tag)::value;
-        constexpr int KB = BUF * KT, SB = BUF * kBlockN * 4;
+        constexpr int KB = BUF * KT, SB = BUF * BN * 4;
+        // On the diagonal, sub-tile st of diagonal block kb holds the keys of query sub-block kb*NST + st: it is
+        // skipped when that is above this wave's rows, masked when equal.  nact = active sub-tiles (wave-uniform).
+        const int gw = wave - kb * NST;                    // sub-tile index that sits on this wave's diagonal
+        const int nact = DIAG ? (gw + 1 < NST ? gw + 1 : NST) : NST;
+        if (DIAG && nact <= 0) return;                     // every key of this block is above the wave's rows
         v4i k_next = k_rsrc, v_next = v_rsrc;
         if (!more) { k_next[2] = 0; v_next[2] = 0; }
         // LDS operand fetches are issued one stage ahead of their MFMAs, in program order pinned by scheduling
@@ -171,7 +180,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         auto load_vfrags = [&](v4i (&vf)[NST], int dt) __attribute__((always_inline)) {
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
-                if (DIAG && st > wave) continue;
+                if (DIAG && st > gw) continue;
                 const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
                     (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[dt] + KB + (32 * st) * D));
                 const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
@@ -183,7 +192,6 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         // Software pipeline inside the wave: the MFMA chain of sub-tile st+1 is issued before the vector work of
         // sub-tile st (the matrix core runs under the wave's own VALU instructions), and LDS operands are requested
         // two stages before the MFMA that consumes them (double-buffered fragments).
-        const int nact = DIAG ? (wave + 1) : NST;          // active sub-tiles (wave-uniform)
         float t[NST][16];
         float mx = -INFINITY;
         v4i fr[2][KS];
@@ -206,7 +214,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         qk_chain(sacc[0], fr[0]);
 #pragma unroll
         for (int st = 0; st < NST; ++st) {
-            if (DIAG && st > wave) {                          // sub-tile entirely above the diagonal
+            if (DIAG && st > gw) {                            // sub-tile entirely above the diagonal
 #pragma unroll
                 for (int r = 0; r < 16; ++r) t[st][r] = -INFINITY;
                 continue;
@@ -219,7 +227,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             __builtin_amdgcn_sched_barrier(0);
             const v16i& acc = sacc[st & 1];
             if (DUMP_S) {
-                int32_t* srow = p.s_dump + ((int64_t)(b * p.heads + h) * p.seqlen + q_row) * p.seqlen + nb * kBlockN + 32 * st;
+                int32_t* srow = p.s_dump + ((int64_t)(b * p.heads + h) * p.seqlen + q_row) * p.seqlen + nb * BN + 32 * st;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) srow[8 * (r >> 2) + 4 * lh + (r & 3)] = acc[r];
             }
@@ -230,7 +238,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                     float x = (float)acc[4 * a4 + b4] * kk[st & 1][a4][b4];
                     if (DIAG) {
                         // position of the key inside the 32x32 tile on the diagonal vs this lane's query
-                        if (st == wave && (8 * a4 + b4) > lq - 4 * lh) x = -INFINITY;
+                        if (st == gw && (8 * a4 + b4) > lq - 4 * lh) x = -INFINITY;
                     }
                     t[st][4 * a4 + b4] = x;
                     mx = fmaxf(mx, x);
@@ -288,7 +296,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             acc = (v16i){0};
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
-                if (DIAG && st > wave) continue;
+                if (DIAG && st > gw) continue;
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[st], p8[st], acc, 0, 0, 0);
             }
         };
@@ -322,8 +330,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             if (DUMP_S || DIAG) issue_loads(nb + 1, BUF ^ 1);      // (a diagonal block is the last one: more == false)
             ks_next = load_ks(nb + 1);
         }
-        compute(buf_tag, diag_tag, nb, more);
-        if (more && tid < kBlockN) *(float*)(smem + ks_wr + (BUF ^ 1) * kBlockN * 4) = cvt_ks(ks_next);
+        compute(buf_tag, diag_tag, nb, more, CAUSAL ? nb - mb * RDIAG : 0);
+        if (more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
     };
 
     // ---- main loop: K/V tiles double-buffered in LDS, one barrier per key block.  The block on the causal
@@ -332,10 +340,10 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         issue_loads(nb_begin, 0);
         {
             const uint32_t s0 = load_ks(nb_begin);
-            if (tid < kBlockN) *(float*)(smem + ks_wr) = cvt_ks(s0);
+            if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
         }
-        const bool has_diag = CAUSAL && (nb_end == mb + 1);
-        const int plain_end = has_diag ? nb_end - 1 : nb_end;
+        const int diag_begin = mb * RDIAG;                 // first key block that touches the diagonal
+        const int plain_end = (CAUSAL && nb_end > diag_begin) ? diag_begin : nb_end;
         int nb = nb_begin;
         while (true) {
             if (nb >= plain_end) break;
@@ -343,9 +351,14 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             if (nb >= plain_end) break;
             step(BoolTag<true>{}, BoolTag<false>{}, nb++);
         }
-        if (CAUSAL && has_diag) {
-            if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb);
-            else step(BoolTag<true>{}, BoolTag<true>{}, nb);
+        if (CAUSAL) {
+#pragma unroll
+            for (int kb = 0; kb < RDIAG; ++kb) {
+                if (nb >= nb_end) break;
+                if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb);
+                else step(BoolTag<true>{}, BoolTag<true>{}, nb);
+                ++nb;
+            }
         }
     }
     if (DUMP_S) return;

@@ -1,0 +1,34 @@
+// Host-side launch functions, one per (variant, head_dim), each defined in its own translation unit so that the
+// kernel instances compile in parallel.
+#pragma once
+#include "intfa_device.h"
+
+namespace intfa {
+
+// Launch switches resolved to template arguments inside the instance files.
+struct LaunchSel {
+    bool causal;
+    int io_dt;       // 0 fp16, 1 bf16 (type of out; also of V / fp Q,K where those are 16-bit)
+    int p_round;     // full-int8 only
+    bool split;      // write split-KV partials instead of the output
+    bool dump_s;     // full-int8 only: export int32 S and stop
+};
+
+template <typename K> inline int launch_kernel(K kernel, const KParams& kp, hipStream_t stream) {
+    const int grid = kp.batch * kp.heads * (kp.seqlen / kBlockM) * kp.num_splits;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, stream, kp);
+    return (int)hipGetLastError();
+}
+
+#define INTFA_DECL_LAUNCH(name) int name(const KParams& kp, const LaunchSel& sel, hipStream_t stream)
+INTFA_DECL_LAUNCH(launch_full_int8_d64);
+INTFA_DECL_LAUNCH(launch_full_int8_d128);
+INTFA_DECL_LAUNCH(launch_full_int8_d256);
+INTFA_DECL_LAUNCH(launch_half_int8_d64);
+INTFA_DECL_LAUNCH(launch_half_int8_d128);
+INTFA_DECL_LAUNCH(launch_half_int8_d256);
+INTFA_DECL_LAUNCH(launch_fp16_d64);
+INTFA_DECL_LAUNCH(launch_fp16_d128);
+INTFA_DECL_LAUNCH(launch_fp16_d256);
+
+}  // namespace intfa

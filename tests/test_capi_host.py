@@ -26,7 +26,9 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in intfa.h but not exported by libintfa.so"
     assert lib.intfa_version() == 1
-    assert lib.intfa_block_n() == 128 == _host.BLOCK
+    assert lib.intfa_fwd_block_n(0, 128) == 128 == _host.BLOCK
+    assert lib.intfa_fwd_block_n(0, 256) == 64 and lib.intfa_fwd_block_n(1, 128) == 64 and lib.intfa_fwd_block_n(2, 64) == 64
+    assert lib.intfa_fwd_block_n(3, 128) < 0 and lib.intfa_fwd_block_n(0, 96) < 0
 
 
 def test_ctypes_struct_matches_c_layout():
