@@ -28,6 +28,18 @@ def max_abs(a, b):
     return (a.float().cpu() - b.float().cpu()).abs().max().item()
 
 
+def assert_same_rounding(o, same):
+    """Kernel against the oracle evaluated with the kernel's own P rounding.  The two differ only through exp2 in the
+    last place, which now and then moves a value of 127 p across a rounding boundary: that one P8 step shows up in a
+    single row as (v8 * v_scale / 127 l) of one key.  So: tight in the mean, tight in nearly every row, and no row
+    beyond the overall bound."""
+    d = (o.float().cpu() - same.float().cpu()).abs()
+    rows = d.amax(dim=-1)
+    assert mean_rel(o, same) <= 2e-4
+    assert d.max().item() <= MAX_ABS
+    assert (rows > 4e-3).float().mean().item() <= 2e-3
+
+
 def quantised(B, H, N, D, seed, dtype=torch.float16, std=1.0, **kw):
     q, k, v, cols = O.make_inputs(B, H, N, D, seed=seed, dtype=dtype, std=std, **kw)
     q8, qs = O.quant_pertoken(q)
@@ -47,7 +59,7 @@ def run_full(x, causal, sm, **kw):
 
 
 # ------------------------------------------------------------------------------------------ int32 S
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [64, 128, 256])
 def test_qk_int32_accumulators_bit_exact(D):
     x = quantised(2, 3, 384, D, seed=5)
     s = M.debug_qk_int32(*gpu(x["q8"], x["k8"])).cpu()
@@ -70,18 +82,22 @@ def test_qk_int32_extreme_values():
     (1, 2, 512, 128, True),
     (2, 3, 384, 64, True),
     (1, 2, 1024, 128, False),
+    (1, 2, 256, 256, False),       # head_dim 256 runs with 64-key blocks
+    (2, 2, 384, 256, True),
 ])
 @pytest.mark.parametrize("p_round", ["rne", "reference"])
 def test_full_int8_matches_oracle(B, H, N, D, causal, p_round):
     x = quantised(B, H, N, D, seed=11)
     sm = D ** -0.5
+    bn = M.block_n("full", D)
+    assert bn == (128 if D <= 128 else 64)
     o = run_full(x, causal, sm, p_round=p_round)
     assert o.dtype == torch.float16 and o.shape == (B, H, N, D) and o.is_contiguous()
-    ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=128)
+    ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=bn)
     assert max_abs(o, ref) <= MAX_ABS and mean_rel(o, ref) <= MEAN_REL
     same = ref if p_round == "reference" else O.attention_full_int8(
-        x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=128, p_requant=O.p_requant_rne)
-    assert max_abs(o, same) <= 4e-3 and mean_rel(o, same) <= 2e-4
+        x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=bn, p_requant=O.p_requant_rne)
+    assert_same_rounding(o, same)
     exact = O.attention_exact(x["q"], x["k"], x["v"], causal, sm)
     assert max_abs(o, exact) <= 6e-2                        # quantisation error itself, reported by the bench
 
@@ -150,6 +166,115 @@ def test_split_kv_matches_oracle_split(causal, splits):
     assert abs(mean_rel(o, single) - mean_rel(ref, single)) <= 1e-3
 
 
+def test_split_kv_head_dim_256():
+    x = quantised(1, 2, 512, 256, seed=18)
+    sm = 256 ** -0.5
+    o = run_full(x, False, sm, num_splits=2, p_round="reference")
+    ref = O.attention_full_int8_splitkv(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], False, sm, 2, block_n=64)
+    assert max_abs(o, ref) <= 4e-3 and mean_rel(o, ref) <= 2e-4
+
+
+# ------------------------------------------------------------------------------------------ half-int8 and fp16
+# No P requantisation on these paths: the only differences from the oracle are fp32 summation order inside the
+# MFMA, the hardware exp2 and where the output is rounded to 16 bits, so the bounds are a few output ulps.
+HALF_FP_CASES = [
+    (1, 4, 256, 64, False, torch.float16),
+    (1, 2, 512, 128, True, torch.float16),
+    (2, 3, 384, 64, True, torch.float16),
+    (1, 2, 256, 256, False, torch.float16),
+    (1, 2, 384, 256, True, torch.float16),
+    (1, 2, 512, 128, True, torch.bfloat16),
+    (2, 2, 256, 64, False, torch.bfloat16),
+]
+
+
+def _ulp_bounds(dtype):
+    return (2e-3, 2e-4) if dtype == torch.float16 else (1.6e-2, 1.5e-3)
+
+
+@pytest.mark.parametrize("B,H,N,D,causal,dtype", HALF_FP_CASES)
+def test_half_int8_matches_oracle(B, H, N, D, causal, dtype):
+    x = quantised(B, H, N, D, seed=31, dtype=dtype)
+    sm = D ** -0.5
+    bn = M.block_n("half", D)
+    o = M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), causal, sm)
+    torch.cuda.synchronize()
+    assert o.dtype == dtype and o.shape == (B, H, N, D)
+    ref = O.attention_int8(x["q8"], x["k8"], x["v"], x["qs"], x["ks"], causal, sm, block_n=bn, out_dtype=dtype)
+    ma, mr = _ulp_bounds(dtype)
+    assert max_abs(o, ref) <= ma and mean_rel(o, ref) <= mr
+    if dtype == torch.float16:
+        exact = O.attention_exact(x["q"], x["k"], x["v"], causal, sm)
+        assert max_abs(o, exact) <= 4e-2 and mean_rel(o, exact) <= 2e-2     # int8 Q/K quantisation error itself
+
+
+@pytest.mark.parametrize("B,H,N,D,causal,dtype", HALF_FP_CASES)
+def test_fp16_attention_matches_oracle(B, H, N, D, causal, dtype):
+    q, k, v, _ = O.make_inputs(B, H, N, D, seed=32, dtype=dtype)
+    sm = D ** -0.5
+    bn = M.block_n("fp", D)
+    o = M.attention(*gpu(q, k, v), causal, sm)
+    torch.cuda.synchronize()
+    assert o.dtype == dtype and o.shape == (B, H, N, D)
+    ref = O.attention_fp(q, k, v, causal, sm, block_n=bn)
+    ma, mr = _ulp_bounds(dtype)
+    assert max_abs(o, ref) <= ma and mean_rel(o, ref) <= mr
+    exact = O.attention_exact(q, k, v, causal, sm)
+    assert max_abs(o, exact) <= (2e-3 if dtype == torch.float16 else 1.6e-2)
+
+
+@pytest.mark.parametrize("d", [16, 32])
+def test_half_and_fp_small_head_dims(d):
+    x = quantised(1, 2, 256, d, seed=33)
+    sm = d ** -0.5
+    o = M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), True, sm)
+    ref = O.attention_int8(x["q8"], x["k8"], x["v"], x["qs"], x["ks"], True, sm, block_n=64)
+    assert o.shape == (1, 2, 256, d) and max_abs(o, ref) <= 2e-3
+    o = M.attention(*gpu(x["q"], x["k"], x["v"]), True, sm)
+    ref = O.attention_fp(x["q"], x["k"], x["v"], True, sm, block_n=64)
+    assert o.shape == (1, 2, 256, d) and max_abs(o, ref) <= 2e-3
+
+
+@pytest.mark.parametrize("variant", ["half", "fp"])
+@pytest.mark.parametrize("causal,splits,D", [(False, 2, 128), (True, 5, 64), (True, 3, 256)])
+def test_half_and_fp_split_kv_equals_single_pass(variant, causal, splits, D):
+    """Without P requantisation the split evaluation is the same sum in another order, except that P is cast to 16 bits
+    relative to another running maximum (an independent 2^-11 relative rounding per element): it must agree with the
+    single pass to a fraction of an output ulp in the mean, and its LSE to fp32 rounding."""
+    x = quantised(1, 2, 1024, D, seed=34)
+    sm = D ** -0.5
+    if variant == "half":
+        args = gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"])
+        f = M.attention_int8
+    else:
+        args = gpu(x["q"], x["k"], x["v"])
+        f = M.attention
+    o1, l1 = f(*args, causal, sm, return_lse=True)
+    o2, l2 = f(*args, causal, sm, num_splits=splits, return_lse=True)
+    torch.cuda.synchronize()
+    assert max_abs(o2, o1) <= 1e-3 and mean_rel(o2, o1) <= 5e-4
+    assert (l1 - l2).abs().max().item() <= 1e-3
+
+
+def test_half_int8_lse_matches_oracle():
+    x = quantised(1, 2, 256, 128, seed=35)
+    _, lse = M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), True, 0.09, return_lse=True)
+    _, ref = O.attention_int8(x["q8"], x["k8"], x["v"], x["qs"], x["ks"], True, 0.09, block_n=64, return_lse=True)
+    assert (lse.cpu() - ref).abs().max().item() < 1e-3
+
+
+def test_three_variants_order_by_precision():
+    """The reference's own evaluation (benchmark/benchmark_int.py: MRE of each variant against fp16 attention): the
+    error against exact attention grows fp16 < half-int8 < full-int8, and every variant stays within a few percent."""
+    x = quantised(1, 4, 1024, 128, seed=36)
+    sm = 128 ** -0.5
+    exact = O.attention_exact(x["q"], x["k"], x["v"], False, sm)
+    e_fp = mean_rel(M.attention(*gpu(x["q"], x["k"], x["v"]), False, sm), exact)
+    e_half = mean_rel(M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), False, sm), exact)
+    e_full = mean_rel(run_full(x, False, sm), exact)
+    assert e_fp < e_half < e_full < 5e-2
+
+
 # ------------------------------------------------------------------------------------------ full-size properties
 def _headline_inputs(B=4, H=32, N=4096, D=128, seed=20):
     g = torch.Generator(device=DEV).manual_seed(seed)
@@ -171,9 +296,12 @@ def test_headline_shape_slices_reproduce_and_v_scale_is_linear():
         sl = lambda t: t[b:b + 1, h:h + 1].contiguous()
         o1 = M.attention_full_int8(sl(q8), sl(k8), sl(v8), sl(qs), sl(ks), sl(vs), False, sm)
         assert torch.equal(o1, o[b:b + 1, h:h + 1])
-    # the value scale is applied once, linearly: doubling it doubles the output exactly (power of two)
+    # the value scale is applied once, linearly: doubling it doubles the output exactly (power of two) wherever the
+    # fp16 result is a normal number; subnormal results are rounded on a fixed 2^-24 grid and may differ by one step
     o2 = M.attention_full_int8(q8, k8, v8, qs, ks, vs * 2, False, sm)
-    assert torch.equal(o2, o * 2)
+    normal = o.abs() > 2.0 ** -14
+    assert torch.equal(o2[normal], (o * 2)[normal])
+    assert (o2.float() - 2 * o.float()).abs().max().item() <= 2.0 ** -24
     # one slice against the CPU oracle at full sequence length
     b, h = 2, 5
     cpu = lambda t: t[b:b + 1, h:h + 1].cpu()
@@ -188,7 +316,41 @@ def test_constant_v_gives_constant_columns_at_full_size():
     v8 = torch.full((B, H, N, D), 64, dtype=torch.int8, device=DEV)
     vs = torch.full((B, H), 1 / 64, dtype=torch.float16, device=DEV)
     o = M.attention_full_int8(q8, k8, v8, qs, ks, vs, True, D ** -0.5)
-    # O = sum(P8) / (127 l): the same for every column of a row, and close to one
+    # O = sum(P8) / (127 l): the same for every column of a row.  Its distance from one is the mass P loses when it is
+    # rounded to multiples of 1/127 (every p below 1/254 becomes zero): a property of the reference's quantisation
+    # that grows with the number of keys, about 0.1 at 4096 keys with these inputs.
     assert torch.equal(o, o[..., :1].expand_as(o))
-    assert (o.float() - 1).abs().max().item() < 0.05
+    assert (o.float() - 1).abs().max().item() < 0.25
     assert torch.equal(o[:, :, 0], torch.ones_like(o[:, :, 0]))    # row 0 sees key 0 only: P8 = 127, l = 1
+
+
+@pytest.mark.parametrize("variant,B,H,N,D,causal", [
+    ("full", 1, 32, 16384, 128, True),      # long-context prefill configuration
+    ("half", 4, 32, 4096, 128, False),
+    ("fp", 4, 32, 4096, 128, False),
+    ("full", 4, 16, 4096, 256, False),      # head_dim 256 configuration
+])
+def test_other_benchmark_shapes_one_slice_against_oracle(variant, B, H, N, D, causal):
+    g = torch.Generator(device=DEV).manual_seed(40)
+    mk = lambda: torch.randn((B, H, N, D), generator=g, device=DEV, dtype=torch.float16)
+    q, k, v = mk(), mk(), mk()
+    sm = D ** -0.5
+    b, h = B - 1, 7
+    cpu = lambda t: t[b:b + 1, h:h + 1].cpu()
+    bn = M.block_n(variant, D)
+    if variant == "fp":
+        o = M.attention(q, k, v, causal, sm)
+        ref = O.attention_fp(cpu(q), cpu(k), cpu(v), causal, sm, block_n=bn)
+    else:
+        q8, qs = M.quant_pertoken(q)
+        k8, ks = M.quant_pertoken(k)
+        if variant == "half":
+            o = M.attention_int8(q8, k8, v, qs, ks, causal, sm)
+            ref = O.attention_int8(cpu(q8), cpu(k8), cpu(v), cpu(qs), cpu(ks), causal, sm, block_n=bn)
+        else:
+            v8, vs = M.quant_pertensor(v)
+            o = M.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm)
+            ref = O.attention_full_int8(cpu(q8), cpu(k8), cpu(v8), cpu(qs), cpu(ks), cpu(vs), causal, sm, block_n=bn,
+                                        p_requant=O.p_requant_rne)
+    assert torch.isfinite(o).all()
+    assert max_abs(o[b:b + 1, h:h + 1], ref) <= 4e-3 and mean_rel(o[b:b + 1, h:h + 1], ref) <= 2e-4
