@@ -21,14 +21,24 @@ INT8_PEAK_TOPS = 5033.0      # MI355X dense int8 MFMA: 256 CUs x 2.4 GHz x 8192 
 FP16_PEAK_TFLOPS = 2516.6
 HBM_PEAK_GBS = 8000.0
 
+# name: variant, B, H, N, D, causal, num_splits, input dtype, std of Q/K/V, fraction of K channels multiplied by 20
 WORKLOADS = {
-    # name: (variant, B, H, N, D, causal, splits)
-    "full_int8_B4_H32_N4096_d128": ("full", 4, 32, 4096, 128, False, 1),
-    "full_int8_B4_H32_N4096_d128_causal": ("full", 4, 32, 4096, 128, True, 1),
-    "half_int8_B8_H32_N2048_d128_causal": ("half", 8, 32, 2048, 128, True, 1),
-    "full_int8_B1_H32_N16384_d128_causal_splitkv": ("full", 1, 32, 16384, 128, True, 2),
-    "full_int8_B16_H16_N1024_d64": ("full", 16, 16, 1024, 64, False, 1),
-    "full_int8_B16_H16_N1024_d256": ("full", 16, 16, 1024, 256, False, 1),
+    "full_int8_B4_H32_N4096_d128": dict(variant="full", B=4, H=32, N=4096, D=128, causal=False, splits=1),
+    "full_int8_B4_H32_N4096_d128_causal": dict(variant="full", B=4, H=32, N=4096, D=128, causal=True, splits=1),
+    "half_int8_B8_H32_N2048_d128_causal": dict(variant="half", B=8, H=32, N=2048, D=128, causal=True, splits=1),
+    "fp16_B4_H32_N4096_d128": dict(variant="fp", B=4, H=32, N=4096, D=128, causal=False, splits=1),
+    "full_int8_B1_H32_N16384_d128_causal_splitkv": dict(variant="full", B=1, H=32, N=16384, D=128, causal=True, splits=2,
+                                                        k_outlier_frac=0.01),
+    "full_int8_B16_H16_N1024_d64_bf16": dict(variant="full", B=16, H=16, N=1024, D=64, causal=False, splits=1,
+                                             dtype="bfloat16", std=0.5),
+    "full_int8_B16_H16_N1024_d256_bf16": dict(variant="full", B=16, H=16, N=1024, D=256, causal=False, splits=1,
+                                              dtype="bfloat16", std=0.5),
+}
+# HBM bytes per launch of the forward kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
+# what the same counter reads for a plain copy of known size; None where not measured.
+MEASURED_TRAFFIC_BYTES = {
+    # FETCH_SIZE 99442.4 x 1.9997 + WRITE_SIZE 131072 x 1.0 (KiB per dispatch): 194.2 MiB read + 128 MiB written
+    "full_int8_B4_H32_N4096_d128": 337848828,
 }
 
 
@@ -68,6 +78,9 @@ def main():
     ap.add_argument("--p-round", default="rne", choices=["rne", "reference"])
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU-baseline budget; 0 skips it")
     ap.add_argument("--no-parity", action="store_true", help="skip the oracle check of one head")
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also run one device-to-device copy of this many MiB before the timed region: a kernel of known "
+                         "HBM traffic that calibrates FETCH_SIZE / WRITE_SIZE when the run is under rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (every (batch, head) is independent; there is no "
@@ -78,26 +91,39 @@ def main():
     import int_flashattention_amd as M
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
-    variant, B, H, N, D, causal, splits = WORKLOADS[args.workload]
+    w = WORKLOADS[args.workload]
+    variant, B, H, N, D, causal, splits = w["variant"], w["B"], w["H"], w["N"], w["D"], w["causal"], w["splits"]
+    dt = getattr(torch, w.get("dtype", "float16"))
+    std = w.get("std", 1.0)
     sm = D ** -0.5
     g = torch.Generator(device=dev).manual_seed(20)
-    dt = torch.float16
-    q = torch.randn((B, H, N, D), generator=g, device=dev, dtype=dt)
-    k = torch.randn((B, H, N, D), generator=g, device=dev, dtype=dt)
-    v = torch.randn((B, H, N, D), generator=g, device=dev, dtype=dt)
-    q8, qs = M.quant_pertoken(q)
-    k8, ks = M.quant_pertoken(k)
-    if variant == "full":
-        v8, vs = M.quant_pertensor(v)
-        step = lambda: M.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, num_splits=splits, p_round=args.p_round)
-    elif variant == "half":
-        step = lambda: M.attention_int8(q8, k8, v, qs, ks, causal, sm, num_splits=splits)
-    else:
+    mk = lambda: (torch.randn((B, H, N, D), generator=g, device=dev, dtype=torch.float32) * std).to(dt)
+    q, k, v = mk(), mk(), mk()
+    outlier_cols = []
+    if w.get("k_outlier_frac"):
+        n_out = max(1, round(w["k_outlier_frac"] * D))
+        outlier_cols = torch.randperm(D, generator=torch.Generator().manual_seed(20))[:n_out].tolist()
+        k[..., outlier_cols] = k[..., outlier_cols] * 20.0
+    bn = M.block_n(variant, D)
+    if variant == "fp":
         step = lambda: M.attention(q, k, v, causal, sm, num_splits=splits)
-    fp_slice = tuple(t[B - 1:B, H - 1:H].cpu() for t in (q, k, v))
-    del q, k
+    else:
+        q8, qs = M.quant_pertoken(q)
+        k8, ks = M.quant_pertoken(k)
+        if variant == "full":
+            v8, vs = M.quant_pertensor(v)
+            step = lambda: M.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, out_dtype=dt, num_splits=splits,
+                                                 p_round=args.p_round)
+        else:
+            step = lambda: M.attention_int8(q8, k8, v, qs, ks, causal, sm, num_splits=splits)
     ops = ops_of(B, H, N, D, causal)
 
+    if args.copy_probe_mib > 0:
+        src = torch.empty((args.copy_probe_mib << 20,), dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -115,43 +141,60 @@ def main():
     achieved = ops / (kern_ms * 1e-3) / 1e12
 
     parity = None
-    if not args.no_parity and variant == "full":
+    if not args.no_parity:
+        # one (batch, head) slice of the timed problem against the CPU oracle run with the kernel's key-block length
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import intfa_oracle as O
         o = step(); torch.cuda.synchronize()
-        b, h, rows = B - 1, H - 1, min(N, 4096)
+        b, h = B - 1, H - 1
         c = lambda t: t[b:b + 1, h:h + 1].cpu()
-        rq = O.p_requant_rne if args.p_round == "rne" else O.p_requant_reference
-        if splits > 1:
-            ref_same = O.attention_full_int8_splitkv(c(q8), c(k8), c(v8), c(qs), c(ks), c(vs), causal, sm, splits, block_n=128)
-            ref = ref_same
-        else:
-            ref_same = O.attention_full_int8(c(q8), c(k8), c(v8), c(qs), c(ks), c(vs), causal, sm, block_n=128, p_requant=rq)
-            ref = O.attention_full_int8(c(q8), c(k8), c(v8), c(qs), c(ks), c(vs), causal, sm, block_n=128)
         got = o[b:b + 1, h:h + 1].float().cpu()
-        exact = O.attention_exact(*fp_slice, causal, sm).float()
-        d1 = (got - ref.float()).abs(); d2 = (got - ref_same.float()).abs(); d3 = (got - exact).abs()
-        d4 = (ref.float() - exact).abs()
-        parity = {"slice": f"batch {b}, head {h}",
-                  "vs_reference_rounding": {"max_abs": d1.max().item(), "mean_rel": (d1.mean() / ref.float().abs().mean()).item()},
-                  "vs_same_rounding": {"max_abs": d2.max().item(), "mean_rel": (d2.mean() / ref_same.float().abs().mean()).item()},
-                  "vs_exact_fp16_attention": {"max_abs": d3.max().item(), "mean_rel": (d3.mean() / exact.abs().mean()).item()},
-                  "oracle_vs_exact_fp16_attention": {"max_abs": d4.max().item(), "mean_rel": (d4.mean() / exact.abs().mean()).item()}}
+        exact = O.attention_exact(c(q), c(k), c(v), causal, sm).float()
+        refs = {}
+        if variant == "full":
+            a8 = (c(q8), c(k8), c(v8), c(qs), c(ks), c(vs), causal, sm)
+            if splits > 1:
+                refs["vs_oracle_split_reference_rounding"] = O.attention_full_int8_splitkv(*a8, splits, block_n=bn, out_dtype=dt)
+            refs["vs_reference_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt)
+            if args.p_round == "rne" and splits == 1:
+                refs["vs_same_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt, p_requant=O.p_requant_rne)
+        elif variant == "half":
+            refs["vs_oracle"] = O.attention_int8(c(q8), c(k8), c(v), c(qs), c(ks), causal, sm, block_n=bn, out_dtype=dt)
+        else:
+            refs["vs_oracle"] = O.attention_fp(c(q), c(k), c(v), causal, sm, block_n=bn)
+        err = lambda x, y: {"max_abs": (x - y).abs().max().item(), "mean_rel": ((x - y).abs().mean() / y.abs().mean()).item()}
+        parity = {"slice": f"batch {b}, head {h}", "oracle_block_n": bn}
+        for name, r in refs.items():
+            parity[name] = err(got, r.float())
+        parity["vs_exact_attention"] = err(got, exact)
+        first = next(iter(refs.values())).float()
+        parity["oracle_vs_exact_attention"] = err(first, exact)
 
+    if variant == "full":
+        peak, peak_model, dtype_s = INT8_PEAK_TOPS, "256 CU x 2.4 GHz x 8192 int8 ops/clk/CU", "int8"
+    elif variant == "half":
+        peak = 1.0 / (0.5 / INT8_PEAK_TOPS + 0.5 / FP16_PEAK_TFLOPS)
+        peak_model, dtype_s = "half of the ops at the int8 rate (5033 T), half at the fp16 rate (2517 T)", "int8+f16"
+    else:
+        peak, peak_model, dtype_s = FP16_PEAK_TFLOPS, "256 CU x 2.4 GHz x 4096 fp16 flops/clk/CU", "f16"
+    kernel_name = "fwd_full_int8_kernel" if variant == "full" else "fwd_f16pv_kernel"
     out = {
         "metric": "attention fwd TOPS + % int8 MFMA peak, B4 H32 N4096 d128 full-int8",
         "value": value, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8" if variant == "full" else ("int8+f16" if variant == "half" else "f16"),
-        "data": "synthetic",
+        "dtype": dtype_s, "data": "synthetic",
         "config": {"workload": args.workload, "variant": variant, "batch": B, "heads": H, "seqlen": N, "head_dim": D,
                    "causal": causal, "num_splits": splits, "p_round": args.p_round, "ops_per_step": ops,
-                   "inputs": "Q,K,V fp16 ~ N(0,1), seed 20; Q,K per-token int8, V per-(batch,head) int8"},
+                   "key_block": bn, "io_dtype": str(dt).replace("torch.", ""),
+                   "inputs": f"Q,K,V {str(dt).replace('torch.', '')} ~ N(0,{std}), seed 20"
+                             + (f", K channels {outlier_cols} x20" if outlier_cols else "")
+                             + ("; Q,K per-token int8" if variant != "fp" else "")
+                             + (", V per-(batch,head) int8" if variant == "full" else "")},
         "pct_int8_peak": 100.0 * value / INT8_PEAK_TOPS,
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": achieved / INT8_PEAK_TOPS, "traffic": None,
-                     "kernel": "fwd_int8_kernel", "avg_launch_ms": kern_ms,
-                     "peak_model": "256 CU x 2.4 GHz x 8192 int8 ops/clk/CU"},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TOP/s" if variant == "full" else "TFLOP/s",
+                     "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel": kernel_name, "avg_launch_ms": kern_ms, "peak_model": peak_model,
+                     "launch_includes": "forward kernel" + (" + split-KV combine kernel" if splits > 1 else "")},
     }
     if parity is not None:
         out["parity"] = parity

@@ -90,6 +90,17 @@ def test_p_requant_reference_exhaustive_over_fp16():
         assert gq == np.trunc(np.float32(np.float16(np.float16(hv * np.float16(127)) + np.float16(0.5))))
 
 
+def test_p_requant_rne_is_round_half_even_of_127p():
+    """The kernels' default rounding: 127*p in fp32, rounded to nearest-even, saturating at 255."""
+    p = np.concatenate([np.linspace(0, 1, 200001, dtype=np.float32), (np.arange(0, 128, dtype=np.float32) + 0.5) / 127])
+    got = O.p_requant_rne(torch.from_numpy(p)).numpy()
+    want = np.clip(np.rint(p * np.float32(127.0)), 0, 255)
+    assert np.array_equal(got, want)
+    assert O.p_requant_rne(torch.tensor([2.5 / 127, 3.5 / 127])).tolist() == [np.rint(np.float32(2.5 / 127) * np.float32(127)),
+                                                                                np.rint(np.float32(3.5 / 127) * np.float32(127))]
+    assert O.p_requant_rne(torch.tensor([3.0])).item() == 255
+
+
 def test_p_requant_modes_differ_by_at_most_one():
     p = torch.linspace(0, 1, 100001)
     d = (O.p_requant_reference(p) - O.p_requant_rne(p)).abs()
