@@ -212,6 +212,9 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
         if (1 < nact) { load_kfrags(fr[1], 1); load_kk(kk[1], 1); }
         __builtin_amdgcn_sched_barrier(0);
         qk_chain(sacc[0], fr[0]);
+        // The MFMAs of sub-tile st+1 are issued one at a time between quarters of the vector work of sub-tile st: each
+        // quarter (4 keys: convert, scale, max) outlasts one MFMA, so the next MFMA of the dependent chain never
+        // stalls the wave at issue and the matrix core runs entirely under this wave's own vector instructions.
 #pragma unroll
         for (int st = 0; st < NST; ++st) {
             if (DIAG && st > gw) {                            // sub-tile entirely above the diagonal
@@ -219,13 +222,12 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
                 for (int r = 0; r < 16; ++r) t[st][r] = -INFINITY;
                 continue;
             }
-            __builtin_amdgcn_sched_barrier(0);
-            if (st + 1 < NST && st + 1 < nact) qk_chain(sacc[(st + 1) & 1], fr[(st + 1) & 1]);
+            const bool next = st + 1 < NST && st + 1 < nact;
             __builtin_amdgcn_sched_barrier(0);
             if (st + 2 < NST && st + 2 < nact) load_kfrags(fr[st & 1], st + 2);
             if (!DUMP_S && !DIAG) issue_k_slice(k_next, nb + 1, BUF ^ 1, st, NST);
-            __builtin_amdgcn_sched_barrier(0);
             const v16i& acc = sacc[st & 1];
+            v16i& nacc = sacc[(st + 1) & 1];
             if (DUMP_S) {
                 int32_t* srow = p.s_dump + ((int64_t)(b * p.heads + h) * p.seqlen + q_row) * p.seqlen + nb * BN + 32 * st;
 #pragma unroll
@@ -233,6 +235,15 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
             }
 #pragma unroll
             for (int a4 = 0; a4 < 4; ++a4) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (next) {
+#pragma unroll
+                    for (int ks = a4 * KS / 4; ks < (a4 + 1) * KS / 4; ++ks) {
+                        if (ks == 0) nacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[(st + 1) & 1][0], qreg[0], (v16i){0}, 0, 0, 0);
+                        else nacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[(st + 1) & 1][ks], qreg[ks], nacc, 0, 0, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int b4 = 0; b4 < 4; ++b4) {
                     float x = (float)acc[4 * a4 + b4] * kk[st & 1][a4][b4];
@@ -302,17 +313,33 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
         };
         __builtin_amdgcn_sched_barrier(0);
         pv_chain(oacc[0], vf[0]);
+        // As in pass 1: the MFMAs of d-tile dt+1 are issued one at a time between quarters of the accumulator update
+        // of d-tile dt.
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             __builtin_amdgcn_sched_barrier(0);
-            if (dt + 1 < DT) pv_chain(oacc[(dt + 1) & 1], vf[(dt + 1) & 1]);
-            __builtin_amdgcn_sched_barrier(0);
             if (dt + 2 < DT) load_vfrags(vf[dt & 1], dt + 2);
             if (!DIAG) issue_v_slice(v_next, nb + 1, BUF ^ 1, dt, DT);
-            __builtin_amdgcn_sched_barrier(0);
+            v16i& nacc = oacc[(dt + 1) & 1];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, (float)oacc[dt & 1][r]);
-
+            for (int a4 = 0; a4 < 4; ++a4) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (dt + 1 < DT) {
+#pragma unroll
+                    for (int st = a4 * NST / 4; st < (a4 + 1) * NST / 4; ++st) {
+                        if (DIAG && st > gw) continue;
+                        if (st == 0) nacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[(dt + 1) & 1][0], p8[0], (v16i){0}, 0, 0, 0);
+                        else nacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[(dt + 1) & 1][st], p8[st], nacc, 0, 0, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) {
+                    const int r = 4 * a4 + b4;
+                    o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, (float)oacc[dt & 1][r]);
+                    asm volatile("" : "+v"(o_acc[dt][r]));     // keeps the update in this slot (it would be sunk below the loop)
+                }
+            }
         }
         l_run = fmaf(l_run, alpha, lsum);
     };
