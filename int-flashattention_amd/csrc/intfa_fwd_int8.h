@@ -273,6 +273,10 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
 #pragma unroll
         for (int st = 0; st < NST; ++st) {
             __builtin_amdgcn_sched_barrier(0);
+            // V of the next block is requested here, well before the end of this block, so that the copy has landed
+            // when the next block waits for it (its buffer was last read before this block's barrier)
+            if (!DIAG) issue_v_slice(v_next, nb + 1, BUF ^ 1, st, NST);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int w4 = 0; w4 < 4; ++w4) {
                 unsigned pk = 0;
@@ -319,7 +323,6 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
         for (int dt = 0; dt < DT; ++dt) {
             __builtin_amdgcn_sched_barrier(0);
             if (dt + 2 < DT) load_vfrags(vf[dt & 1], dt + 2);
-            if (!DIAG) issue_v_slice(v_next, nb + 1, BUF ^ 1, dt, DT);
             v16i& nacc = oacc[(dt + 1) & 1];
 #pragma unroll
             for (int a4 = 0; a4 < 4; ++a4) {
