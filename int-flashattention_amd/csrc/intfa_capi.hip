@@ -130,6 +130,7 @@ int run_forward(int variant, const intfa_fwd_params* p, int qk_bytes, int v_byte
     if (variant == INTFA_VARIANT_FULL_INT8 && p->p_round != INTFA_PROUND_RNE && p->p_round != INTFA_PROUND_REFERENCE) return INTFA_ERR_DTYPE;
     rc = setup_split(p, block_n_for(variant, kp.head_dim), &kp);
     if (rc != INTFA_OK) return rc;
+    kp.pair_mblocks = (kp.causal && kp.num_splits <= 1 && (kp.seqlen / kBlockM) % 2 == 0) ? 1 : 0;
     rc = dispatch(variant, p, kp, false, stream);
     if (rc != INTFA_OK || kp.num_splits <= 1) return rc;
     return launch_combine(p, kp, stream);

@@ -47,7 +47,10 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     // L2; give every XCD whole heads so that the K/V tiles of a head are re-read from one L2.
     const int n_mblk = p.seqlen / kBlockM;
     const int n_split = SPLIT ? p.num_splits : 1;
-    const int per_head = n_mblk * n_split;
+    // Causal single-pass launches pair query block i with query block n-1-i in one workgroup (heavy one first): every
+    // workgroup then walks the same number of key blocks and the launch has no tail of light workgroups.
+    const bool pair = CAUSAL && !SPLIT && p.pair_mblocks != 0;
+    const int per_head = pair ? n_mblk / 2 : n_mblk * n_split;
     const int n_heads = p.batch * p.heads;
     const int bid = blockIdx.x;
     int head, rem;
@@ -59,9 +62,14 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
         head = bid / per_head;
         rem = bid % per_head;
     }
-    int mb = rem / n_split;
+    const int mb_idx = rem / n_split;
     const int split = rem % n_split;
-    if (CAUSAL) mb = n_mblk - 1 - mb;            // heaviest query blocks first
+    const int njobs = pair ? 2 : 1;
+#pragma clang loop unroll(disable)
+    for (int job = 0; job < njobs; ++job) {
+    if (job) __syncthreads();                    // every wave is done with the LDS tiles of the first query block
+    int mb = mb_idx;
+    if (CAUSAL) mb = (pair && job) ? mb_idx : n_mblk - 1 - mb_idx;     // heaviest query blocks first
     const int b = head / p.heads, h = head % p.heads;
 
     // key-block range of this workgroup
@@ -439,6 +447,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
             }
         }
     if (pe->lse != nullptr && lh == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
+    }   // job
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
