@@ -131,6 +131,22 @@ int intfa_fwd_fp16(const intfa_fwd_params* p, void* stream);
  * Uses q, k and their strides, batch, heads, seqlen, head_dim of the block. */
 int intfa_debug_qk_int32(const intfa_fwd_params* p, int32_t* s_out, void* stream);
 
+/* quant_pertoken(X) -> (int8 X, scale) of the reference's harness (benchmark.py:96-100): per row of head_dim
+ * elements, scale = absmax / 127 and q = round(x / scale), every step evaluated in x's 16-bit type as torch does.
+ * x: [batch, heads, seqlen, head_dim] fp16 or bf16 (dtype = INTFA_F16 / INTFA_BF16), strides in elements, head_dim
+ * contiguous and one of 16, 32, 64, 128, 256; q8: int8, written contiguous; scale: [batch, heads, seqlen] in x's
+ * type, contiguous. */
+int intfa_quant_pertoken(const void* x, int64_t stride_b, int64_t stride_h, int64_t stride_n, void* q8, void* scale,
+                         int32_t batch, int32_t heads, int32_t seqlen, int32_t head_dim, int32_t dtype, void* stream);
+
+/* quant_pertensor(X) -> (int8 X, scale) (benchmark.py:102-107): one scale per (batch, head) slice; scale is
+ * [batch, heads] in x's type.  Needs intfa_quant_pertensor_workspace_bytes() bytes of device scratch (4-byte
+ * aligned) for the per-slice maxima. */
+size_t intfa_quant_pertensor_workspace_bytes(int32_t batch, int32_t heads);
+int intfa_quant_pertensor(const void* x, int64_t stride_b, int64_t stride_h, int64_t stride_n, void* q8, void* scale,
+                          int32_t batch, int32_t heads, int32_t seqlen, int32_t head_dim, int32_t dtype,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -36,7 +36,8 @@ class FwdParams(ctypes.Structure):
 VARIANT_FULL_INT8, VARIANT_HALF_INT8, VARIANT_FP16 = 0, 1, 2
 
 EXPORTS = ("intfa_version", "intfa_error_string", "intfa_fwd_block_n", "intfa_fwd_workspace_bytes",
-           "intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16", "intfa_debug_qk_int32")
+           "intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16", "intfa_debug_qk_int32",
+           "intfa_quant_pertoken", "intfa_quant_pertensor_workspace_bytes", "intfa_quant_pertensor")
 
 _lib = None
 
@@ -66,6 +67,13 @@ def load():
         fn.argtypes = [pp, ctypes.c_void_p]
     lib.intfa_debug_qk_int32.restype = ctypes.c_int
     lib.intfa_debug_qk_int32.argtypes = [pp, ctypes.c_void_p, ctypes.c_void_p]
+    i64, i32, vp = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p
+    lib.intfa_quant_pertoken.restype = ctypes.c_int
+    lib.intfa_quant_pertoken.argtypes = [vp, i64, i64, i64, vp, vp, i32, i32, i32, i32, i32, vp]
+    lib.intfa_quant_pertensor_workspace_bytes.restype = ctypes.c_size_t
+    lib.intfa_quant_pertensor_workspace_bytes.argtypes = [i32, i32]
+    lib.intfa_quant_pertensor.restype = ctypes.c_int
+    lib.intfa_quant_pertensor.argtypes = [vp, i64, i64, i64, vp, vp, i32, i32, i32, i32, i32, vp, ctypes.c_size_t, vp]
     _lib = lib
     return lib
 

@@ -1,0 +1,207 @@
+// Symmetric int8 quantisers of the attention inputs (benchmark.py:96-107) as HBM-bound streaming kernels.
+//
+// Arithmetic follows the reference's torch expressions evaluated in the input's 16-bit type, operation by
+// operation (each torch op on fp16/bf16 computes in fp32 and rounds the result to the 16-bit type):
+//     scale = absmax / 127                      -> fp32 division, rounded to the 16-bit type
+//     q     = round(x / scale).to(int8)         -> fp32 division rounded to the 16-bit type, round-half-even,
+//                                                  integer conversion truncated to 8 bits
+// Layout: x is [B, H, N, d] with arbitrary batch/head/row strides and contiguous d; q8 is written contiguous; a lane
+// owns 8 consecutive elements (one 16-byte load, one 8-byte store) and d / 8 lanes share a row.
+#include "../../include/intfa.h"
+#include "intfa_device.h"
+
+using namespace intfa;
+
+namespace {
+
+template <int DT> __device__ __forceinline__ float to_f32(uint16_t bits) {
+    if (DT == 0) return (float)__builtin_bit_cast(_Float16, bits);
+    return __builtin_bit_cast(float, (uint32_t)bits << 16);
+}
+template <int DT> __device__ __forceinline__ uint16_t from_f32(float f) {      // round-to-nearest-even
+    if (DT == 0) return __builtin_bit_cast(uint16_t, (_Float16)f);
+    return (uint16_t)f32_to_bf16_bits(f);
+}
+// |x| of a 16-bit float as an unsigned integer: monotonic in |x| for finite values, so max works on the bits
+__device__ __forceinline__ uint32_t abs_bits(uint16_t b) { return b & 0x7fffu; }
+
+// round(x / scale) truncated to int8, both operands and the quotient in the 16-bit type
+template <int DT> __device__ __forceinline__ int quant_one(uint16_t xb, float scale) {
+    const float q16 = to_f32<DT>(from_f32<DT>(to_f32<DT>(xb) / scale));
+    const float r = __builtin_rintf(q16);
+    return (r == r) ? (int)r : 0;                                               // NaN (zero row) -> 0
+}
+
+template <int DT> __device__ __forceinline__ void quant_store8(const v4i raw, float scale, char* dst) {
+    int out[2];
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+        uint32_t pk = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t word = (uint32_t)raw[2 * w + j / 2];
+            const uint16_t xb = (uint16_t)(j & 1 ? word >> 16 : word & 0xffffu);
+            pk |= ((uint32_t)quant_one<DT>(xb, scale) & 0xffu) << (8 * j);
+        }
+        out[w] = (int)pk;
+    }
+    *(v2i*)dst = (v2i){out[0], out[1]};
+}
+
+__device__ __forceinline__ uint32_t amax8(const v4i raw) {
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w = (uint32_t)raw[i];
+        const uint32_t a = abs_bits((uint16_t)(w & 0xffffu)), b = abs_bits((uint16_t)(w >> 16));
+        m = m > a ? m : a;
+        m = m > b ? m : b;
+    }
+    return m;
+}
+
+struct QuantParams {
+    const char* x; char* q8; char* scale; uint32_t* amax;
+    int64_t sb, sh, sn;             // bytes
+    int32_t heads, seqlen, head_dim;
+    int64_t rows;                   // batch * heads * seqlen
+};
+
+// ---- per token: LPR = d / 8 lanes per row, reduction of the row maximum inside those lanes
+template <int DT, int LPR> __global__ void __launch_bounds__(256) quant_pertoken_kernel(const QuantParams p) {
+    constexpr int RPB = 256 / LPR;                       // rows per workgroup pass
+    const int sub = threadIdx.x % LPR, rl = threadIdx.x / LPR;
+    for (int64_t row = (int64_t)blockIdx.x * RPB + rl; row < p.rows; row += (int64_t)gridDim.x * RPB) {
+        const int64_t n = row % p.seqlen, bh = row / p.seqlen;
+        const int64_t h = bh % p.heads, b = bh / p.heads;
+        const v4i raw = *(const v4i*)(p.x + b * p.sb + h * p.sh + n * p.sn + sub * 16);
+        uint32_t m = amax8(raw);
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) {
+            const uint32_t o = (uint32_t)__shfl_xor((int)m, off, 64);
+            m = m > o ? m : o;
+        }
+        const uint16_t sbits = from_f32<DT>(to_f32<DT>((uint16_t)m) / 127.0f);
+        if (sub == 0) ((uint16_t*)p.scale)[row] = sbits;
+        quant_store8<DT>(raw, to_f32<DT>(sbits), p.q8 + row * p.head_dim + sub * 8);
+    }
+}
+
+// ---- per (batch, head): maximum over the whole [N, d] slice in two launches
+__global__ void quant_clear_kernel(uint32_t* amax, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) amax[i] = 0u;
+}
+
+template <int LPR> __global__ void __launch_bounds__(256) quant_slice_amax_kernel(const QuantParams p, int chunks) {
+    constexpr int RPB = 256 / LPR;
+    const int sub = threadIdx.x % LPR, rl = threadIdx.x / LPR;
+    const int bh = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
+    const int64_t h = bh % p.heads, b = bh / p.heads;
+    const char* base = p.x + b * p.sb + h * p.sh + sub * 16;
+    uint32_t m = 0;
+    for (int n = chunk * RPB + rl; n < p.seqlen; n += chunks * RPB) {
+        const uint32_t r = amax8(*(const v4i*)(base + (int64_t)n * p.sn));
+        m = m > r ? m : r;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)m, off, 64);
+        m = m > o ? m : o;
+    }
+    if ((threadIdx.x & 63) == 0) atomicMax(p.amax + bh, m);
+}
+
+template <int DT, int LPR> __global__ void __launch_bounds__(256) quant_slice_apply_kernel(const QuantParams p) {
+    constexpr int RPB = 256 / LPR;
+    const int sub = threadIdx.x % LPR, rl = threadIdx.x / LPR;
+    for (int64_t row = (int64_t)blockIdx.x * RPB + rl; row < p.rows; row += (int64_t)gridDim.x * RPB) {
+        const int64_t n = row % p.seqlen, bh = row / p.seqlen;
+        const int64_t h = bh % p.heads, b = bh / p.heads;
+        const uint16_t sbits = from_f32<DT>(to_f32<DT>((uint16_t)p.amax[bh]) / 127.0f);
+        if (n == 0 && sub == 0) ((uint16_t*)p.scale)[bh] = sbits;
+        const v4i raw = *(const v4i*)(p.x + b * p.sb + h * p.sh + n * p.sn + sub * 16);
+        quant_store8<DT>(raw, to_f32<DT>(sbits), p.q8 + row * p.head_dim + sub * 8);
+    }
+}
+
+int check(const void* x, const void* q8, const void* scale, int64_t sb, int64_t sh, int64_t sn, int batch, int heads,
+          int seqlen, int head_dim, int dtype, QuantParams* qp) {
+    if (x == nullptr || q8 == nullptr || scale == nullptr) return INTFA_ERR_NULL;
+    if (batch <= 0 || heads <= 0 || seqlen <= 0) return INTFA_ERR_SHAPE;
+    if (head_dim != 16 && head_dim != 32 && head_dim != 64 && head_dim != 128 && head_dim != 256) return INTFA_ERR_HEAD_DIM;
+    if (dtype != INTFA_F16 && dtype != INTFA_BF16) return INTFA_ERR_DTYPE;
+    if ((reinterpret_cast<uintptr_t>(x) & 15u) || (reinterpret_cast<uintptr_t>(q8) & 7u) || (reinterpret_cast<uintptr_t>(scale) & 1u))
+        return INTFA_ERR_ALIGN;
+    if ((sb * 2) % 16 || (sh * 2) % 16 || (sn * 2) % 16) return INTFA_ERR_ALIGN;
+    qp->x = (const char*)x; qp->q8 = (char*)q8; qp->scale = (char*)scale; qp->amax = nullptr;
+    qp->sb = sb * 2; qp->sh = sh * 2; qp->sn = sn * 2;
+    qp->heads = heads; qp->seqlen = seqlen; qp->head_dim = head_dim;
+    qp->rows = (int64_t)batch * heads * seqlen;
+    return INTFA_OK;
+}
+
+int grid_for(int64_t rows, int rows_per_block) {
+    const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+    const int64_t cap = 256 * 16;                        // a few waves of workgroups per CU, grid-stride beyond
+    return (int)(blocks < cap ? blocks : cap);
+}
+
+}  // namespace
+
+#define INTFA_LPR_SWITCH(d, CALL)            \
+    switch (d) {                             \
+        case 16: CALL(2); break;             \
+        case 32: CALL(4); break;             \
+        case 64: CALL(8); break;             \
+        case 128: CALL(16); break;           \
+        default: CALL(32); break;            \
+    }
+
+extern "C" {
+
+int intfa_quant_pertoken(const void* x, int64_t stride_b, int64_t stride_h, int64_t stride_n, void* q8, void* scale,
+                         int32_t batch, int32_t heads, int32_t seqlen, int32_t head_dim, int32_t dtype, void* stream) {
+    QuantParams qp;
+    const int rc = check(x, q8, scale, stride_b, stride_h, stride_n, batch, heads, seqlen, head_dim, dtype, &qp);
+    if (rc != INTFA_OK) return rc;
+    hipStream_t st = (hipStream_t)stream;
+#define INTFA_CALL(LPR) do { const int g = grid_for(qp.rows, 256 / LPR); \
+        if (dtype == INTFA_F16) hipLaunchKernelGGL((quant_pertoken_kernel<0, LPR>), dim3(g), dim3(256), 0, st, qp); \
+        else hipLaunchKernelGGL((quant_pertoken_kernel<1, LPR>), dim3(g), dim3(256), 0, st, qp); } while (0)
+    INTFA_LPR_SWITCH(head_dim, INTFA_CALL)
+#undef INTFA_CALL
+    return (int)hipGetLastError();
+}
+
+size_t intfa_quant_pertensor_workspace_bytes(int32_t batch, int32_t heads) {
+    return (batch > 0 && heads > 0) ? (size_t)batch * heads * sizeof(uint32_t) : 0;
+}
+
+int intfa_quant_pertensor(const void* x, int64_t stride_b, int64_t stride_h, int64_t stride_n, void* q8, void* scale,
+                          int32_t batch, int32_t heads, int32_t seqlen, int32_t head_dim, int32_t dtype,
+                          void* workspace, size_t workspace_bytes, void* stream) {
+    QuantParams qp;
+    const int rc = check(x, q8, scale, stride_b, stride_h, stride_n, batch, heads, seqlen, head_dim, dtype, &qp);
+    if (rc != INTFA_OK) return rc;
+    if (workspace == nullptr || workspace_bytes < intfa_quant_pertensor_workspace_bytes(batch, heads) ||
+        (reinterpret_cast<uintptr_t>(workspace) & 3u)) return INTFA_ERR_WORKSPACE;
+    qp.amax = (uint32_t*)workspace;
+    hipStream_t st = (hipStream_t)stream;
+    const int slices = batch * heads;
+    hipLaunchKernelGGL(quant_clear_kernel, dim3((slices + 255) / 256), dim3(256), 0, st, qp.amax, slices);
+#define INTFA_CALL(LPR) do { \
+        const int rpb = 256 / LPR; \
+        int chunks = (seqlen + rpb - 1) / rpb; \
+        const int want = (256 * 8 + slices - 1) / slices;          /* about 8 workgroups per CU over all slices */ \
+        if (chunks > want) chunks = want; \
+        hipLaunchKernelGGL((quant_slice_amax_kernel<LPR>), dim3(slices * chunks), dim3(256), 0, st, qp, chunks); \
+        const int g = grid_for(qp.rows, rpb); \
+        if (dtype == INTFA_F16) hipLaunchKernelGGL((quant_slice_apply_kernel<0, LPR>), dim3(g), dim3(256), 0, st, qp); \
+        else hipLaunchKernelGGL((quant_slice_apply_kernel<1, LPR>), dim3(g), dim3(256), 0, st, qp); } while (0)
+    INTFA_LPR_SWITCH(head_dim, INTFA_CALL)
+#undef INTFA_CALL
+    return (int)hipGetLastError();
+}
+
+}  // extern "C"

@@ -114,9 +114,22 @@ def test_entry_points_keep_the_reference_asserts():
         M.attention_full_int8(q, q, q, s, s, torch.ones((1, 1), dtype=torch.float16), False, 1.0)
 
 
-def test_package_quantisers_match_the_oracle():
-    import intfa_oracle as O
-    x = torch.randn((2, 3, 16, 32), generator=torch.Generator().manual_seed(0)).half()
-    for mine, ref in ((M.quant_pertoken, O.quant_pertoken), (M.quant_pertensor, O.quant_pertensor)):
-        a, sa = mine(x); b, sb = ref(x)
-        assert torch.equal(a, b) and torch.equal(sa, sb)
+def test_quantisers_refuse_cpu_tensors_and_bad_arguments():
+    x = torch.randn((2, 3, 16, 32)).half()
+    for fn in (M.quant_pertoken, M.quant_pertensor):
+        with pytest.raises(RuntimeError, match="GPU only"):     # no CPU fallback
+            fn(x)
+    lib = _capi.load()
+    one = ctypes.c_void_p(16)            # a non-null, 16-byte aligned address: validation happens before any launch
+    ok = dict(x=one, sb=96 * 32, sh=32 * 32, sn=32, q8=one, scale=one, B=2, H=3, N=32, d=32, dt=_capi.INTFA_F16)
+
+    def call(**kw):
+        a = dict(ok, **kw)
+        return lib.intfa_quant_pertoken(a["x"], a["sb"], a["sh"], a["sn"], a["q8"], a["scale"], a["B"], a["H"], a["N"], a["d"],
+                                        a["dt"], None)
+    assert call(x=None) == -1 and call(q8=None) == -1 and call(scale=None) == -1
+    assert call(d=48) == -2 and call(dt=_capi.INTFA_F32) == -5 and call(B=0) == -7
+    assert call(sn=33) == -4 and call(x=ctypes.c_void_p(8)) == -4
+    assert lib.intfa_quant_pertensor_workspace_bytes(4, 32) == 4 * 32 * 4
+    rc = lib.intfa_quant_pertensor(one, 96 * 32, 32 * 32, 32, one, one, 2, 3, 32, 32, _capi.INTFA_F16, None, 0, None)
+    assert rc == -6
