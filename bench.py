@@ -33,6 +33,9 @@ WORKLOADS = {
                                              dtype="bfloat16", std=0.5),
     "full_int8_B16_H16_N1024_d256_bf16": dict(variant="full", B=16, H=16, N=1024, D=256, causal=False, splits=1,
                                               dtype="bfloat16", std=0.5),
+    # the input quantisers (HBM-bound): Q/K per token, V per (batch, head)
+    "quant_pertoken_B4_H32_N4096_d128": dict(variant="quant_token", B=4, H=32, N=4096, D=128, causal=False, splits=1),
+    "quant_pertensor_B4_H32_N4096_d128": dict(variant="quant_tensor", B=4, H=32, N=4096, D=128, causal=False, splits=1),
 }
 # HBM bytes per launch of the forward kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
 # what the same counter reads for a plain copy of known size; None where not measured.
@@ -67,6 +70,36 @@ def cpu_baseline(budget_s: float):
     return {"value": ops_of(B, H, N, D, False) / med / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(),
             "kind": "port", "ms": med * 1e3,
             "sample": f"{len(times)} runs of the PyTorch CPU oracle, full-int8 B{B} H{H} N{N} d{D} non-causal, median"}
+
+
+def bench_quant(args, variant, x, B, H, N, D, dt):
+    """Times one quantiser; algorithmic bytes = 2 per element read + 1 written (+ scales); the per-(batch, head) variant
+    reads its input twice (maximum, then quantise)."""
+    import torch
+    import int_flashattention_amd as M
+    fn = M.quant_pertoken if variant == "quant_token" else M.quant_pertensor
+    n = B * H * N * D
+    alg_bytes = (2 + 1) * n + (2 * B * H * N if variant == "quant_token" else 2 * B * H) + (2 * n if variant == "quant_tensor" else 0)
+    for _ in range(args.warmup):
+        fn(x)
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for e0, e1 in evs:
+        e0.record(); fn(x); e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kern_ms = statistics.fmean(e0.elapsed_time(e1) for e0, e1 in evs)
+    ms_step = wall * 1e3 / args.steps
+    out = {"metric": "input quantiser throughput (algorithmic HBM bytes per second)", "value": alg_bytes / (ms_step * 1e-3) / 1e9,
+           "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16->int8", "data": "synthetic",
+           "config": {"workload": args.workload, "batch": B, "heads": H, "seqlen": N, "head_dim": D, "bytes_per_step": alg_bytes},
+           "roofline": {"bound": "hbm", "achieved": alg_bytes / (kern_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": alg_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                        "kernel": "quant_pertoken_kernel" if variant == "quant_token" else "quant_slice_amax_kernel + quant_slice_apply_kernel",
+                        "avg_launch_ms": kern_ms}}
+    print(json.dumps(out))
 
 
 def main():
@@ -104,6 +137,8 @@ def main():
         n_out = max(1, round(w["k_outlier_frac"] * D))
         outlier_cols = torch.randperm(D, generator=torch.Generator().manual_seed(20))[:n_out].tolist()
         k[..., outlier_cols] = k[..., outlier_cols] * 20.0
+    if variant.startswith("quant"):
+        return bench_quant(args, variant, q, B, H, N, D, dt)
     bn = M.block_n(variant, D)
     if variant == "fp":
         step = lambda: M.attention(q, k, v, causal, sm, num_splits=splits)

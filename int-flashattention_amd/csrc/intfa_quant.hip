@@ -68,22 +68,43 @@ struct QuantParams {
 };
 
 // ---- per token: LPR = d / 8 lanes per row, reduction of the row maximum inside those lanes
+constexpr int kRowsInFlight = 4;    // independent 16-byte loads a lane has in flight (HBM latency x bandwidth needs several)
+
+// rows are numbered (batch, head, position) in that order; the count fits 31 bits (checked on the host), so the index
+// arithmetic is 32-bit
+__device__ __forceinline__ const char* row_ptr(const QuantParams& p, uint32_t row, int sub, uint32_t* bh_out) {
+    const uint32_t bh = row / (uint32_t)p.seqlen, n = row - bh * (uint32_t)p.seqlen;
+    const uint32_t b = bh / (uint32_t)p.heads, h = bh - b * (uint32_t)p.heads;
+    *bh_out = bh;
+    return p.x + b * p.sb + h * p.sh + n * p.sn + sub * 16;
+}
+
 template <int DT, int LPR> __global__ void __launch_bounds__(256) quant_pertoken_kernel(const QuantParams p) {
-    constexpr int RPB = 256 / LPR;                       // rows per workgroup pass
+    constexpr int RPB = 256 / LPR;                       // rows per workgroup step
     const int sub = threadIdx.x % LPR, rl = threadIdx.x / LPR;
-    for (int64_t row = (int64_t)blockIdx.x * RPB + rl; row < p.rows; row += (int64_t)gridDim.x * RPB) {
-        const int64_t n = row % p.seqlen, bh = row / p.seqlen;
-        const int64_t h = bh % p.heads, b = bh / p.heads;
-        const v4i raw = *(const v4i*)(p.x + b * p.sb + h * p.sh + n * p.sn + sub * 16);
-        uint32_t m = amax8(raw);
+    const uint32_t step = gridDim.x * RPB, rows = (uint32_t)p.rows;
+    for (uint32_t row0 = blockIdx.x * RPB + rl; row0 < rows; row0 += step * kRowsInFlight) {
+        v4i raw[kRowsInFlight];
 #pragma unroll
-        for (int off = LPR / 2; off > 0; off >>= 1) {
-            const uint32_t o = (uint32_t)__shfl_xor((int)m, off, 64);
-            m = m > o ? m : o;
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const uint32_t row = row0 + u * step;
+            uint32_t bh;
+            raw[u] = row < rows ? *(const v4i*)row_ptr(p, row, sub, &bh) : (v4i){0, 0, 0, 0};
         }
-        const uint16_t sbits = from_f32<DT>(to_f32<DT>((uint16_t)m) / 127.0f);
-        if (sub == 0) ((uint16_t*)p.scale)[row] = sbits;
-        quant_store8<DT>(raw, to_f32<DT>(sbits), p.q8 + row * p.head_dim + sub * 8);
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const uint32_t row = row0 + u * step;
+            uint32_t m = amax8(raw[u]);
+#pragma unroll
+            for (int off = LPR / 2; off > 0; off >>= 1) {
+                const uint32_t o = (uint32_t)__shfl_xor((int)m, off, 64);
+                m = m > o ? m : o;
+            }
+            if (row >= rows) continue;
+            const uint16_t sbits = from_f32<DT>(to_f32<DT>((uint16_t)m) / 127.0f);
+            if (sub == 0) ((uint16_t*)p.scale)[row] = sbits;
+            quant_store8<DT>(raw[u], to_f32<DT>(sbits), p.q8 + (int64_t)row * p.head_dim + sub * 8);
+        }
     }
 }
 
@@ -100,9 +121,19 @@ template <int LPR> __global__ void __launch_bounds__(256) quant_slice_amax_kerne
     const int64_t h = bh % p.heads, b = bh / p.heads;
     const char* base = p.x + b * p.sb + h * p.sh + sub * 16;
     uint32_t m = 0;
-    for (int n = chunk * RPB + rl; n < p.seqlen; n += chunks * RPB) {
-        const uint32_t r = amax8(*(const v4i*)(base + (int64_t)n * p.sn));
-        m = m > r ? m : r;
+    const int nstep = chunks * RPB;
+    for (int n0 = chunk * RPB + rl; n0 < p.seqlen; n0 += nstep * kRowsInFlight) {
+        v4i raw[kRowsInFlight];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const int n = n0 + u * nstep;
+            raw[u] = n < p.seqlen ? *(const v4i*)(base + (int64_t)n * p.sn) : (v4i){0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const uint32_t r = amax8(raw[u]);
+            m = m > r ? m : r;
+        }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -115,13 +146,24 @@ template <int LPR> __global__ void __launch_bounds__(256) quant_slice_amax_kerne
 template <int DT, int LPR> __global__ void __launch_bounds__(256) quant_slice_apply_kernel(const QuantParams p) {
     constexpr int RPB = 256 / LPR;
     const int sub = threadIdx.x % LPR, rl = threadIdx.x / LPR;
-    for (int64_t row = (int64_t)blockIdx.x * RPB + rl; row < p.rows; row += (int64_t)gridDim.x * RPB) {
-        const int64_t n = row % p.seqlen, bh = row / p.seqlen;
-        const int64_t h = bh % p.heads, b = bh / p.heads;
-        const uint16_t sbits = from_f32<DT>(to_f32<DT>((uint16_t)p.amax[bh]) / 127.0f);
-        if (n == 0 && sub == 0) ((uint16_t*)p.scale)[bh] = sbits;
-        const v4i raw = *(const v4i*)(p.x + b * p.sb + h * p.sh + n * p.sn + sub * 16);
-        quant_store8<DT>(raw, to_f32<DT>(sbits), p.q8 + row * p.head_dim + sub * 8);
+    const uint32_t step = gridDim.x * RPB, rows = (uint32_t)p.rows;
+    for (uint32_t row0 = blockIdx.x * RPB + rl; row0 < rows; row0 += step * kRowsInFlight) {
+        v4i raw[kRowsInFlight];
+        uint32_t bh[kRowsInFlight];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const uint32_t row = row0 + u * step;
+            bh[u] = 0;
+            raw[u] = row < rows ? *(const v4i*)row_ptr(p, row, sub, &bh[u]) : (v4i){0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const uint32_t row = row0 + u * step;
+            if (row >= rows) continue;
+            const uint16_t sbits = from_f32<DT>(to_f32<DT>((uint16_t)p.amax[bh[u]]) / 127.0f);
+            if (row == bh[u] * (uint32_t)p.seqlen && sub == 0) ((uint16_t*)p.scale)[bh[u]] = sbits;
+            quant_store8<DT>(raw[u], to_f32<DT>(sbits), p.q8 + (int64_t)row * p.head_dim + sub * 8);
+        }
     }
 }
 
@@ -138,12 +180,13 @@ int check(const void* x, const void* q8, const void* scale, int64_t sb, int64_t 
     qp->sb = sb * 2; qp->sh = sh * 2; qp->sn = sn * 2;
     qp->heads = heads; qp->seqlen = seqlen; qp->head_dim = head_dim;
     qp->rows = (int64_t)batch * heads * seqlen;
+    if (qp->rows >= (1ll << 31) - (1 << 24)) return INTFA_ERR_SHAPE;      // 32-bit row indices, with room for the strides
     return INTFA_OK;
 }
 
 int grid_for(int64_t rows, int rows_per_block) {
     const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-    const int64_t cap = 256 * 16;                        // a few waves of workgroups per CU, grid-stride beyond
+    const int64_t cap = 256 * 8;                         // every CU full (8 workgroups of 256 threads), grid-stride beyond
     return (int)(blocks < cap ? blocks : cap);
 }
 
