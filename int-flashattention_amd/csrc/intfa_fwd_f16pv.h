@@ -149,13 +149,59 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     const uint32_t ks_rd = OFF_KS + 16 * lh;
     const uint32_t ks_wr = OFF_KS + 4 * (tid & (BN - 1));
 
+    auto mfma16 = [&](v4i a, v4i b, v16f c) __attribute__((always_inline)) -> v16f {
+        if (IO_DT == 0) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+    };
+
+    // One key block out of LDS buffer BUF.  Inside the wave the work is software-pipelined and pinned with scheduling
+    // barriers: the MFMAs of S^T sub-tile st+1 are issued one at a time between quarters of the vector work of sub-tile
+    // st, the MFMAs of output d-tile dt between quarters of the rescaling of d-tile dt+1, and LDS operands are requested
+    // one or two stages before the MFMA that consumes them.
     auto compute = [&](auto buf_tag, auto diag_tag, int nb, int kb) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         constexpr bool DIAG = decltype(diag_tag)::value;
         constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4;
+        static_assert(NST == 2, "the quarter interleave below assumes two sub-tiles of 32 keys");
         const int gw = wave - kb * NST;                 // sub-tile on this wave's diagonal (DIAG only)
         if (DIAG && gw < 0) return;                     // block entirely above the wave's rows
-        // -------- S^T sub-tiles and running max
+        const int nact = DIAG ? (gw + 1 < NST ? gw + 1 : NST) : NST;
+        // -------- operands of both S^T sub-tiles
+        v4i fr[NST][KS];
+        v4f kk[NST][4];
+#pragma unroll
+        for (int st = 0; st < NST; ++st) {
+            if (DIAG && st > gw) continue;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) fr[st][ks] = *(const v4i*)(smem + k_rd[ks] + KB + 32 * st * KROW);
+            if (QK_INT8) {
+#pragma unroll
+                for (int a4 = 0; a4 < 4; ++a4) kk[st][a4] = *(const v4f*)(smem + ks_rd + SB + 4 * (32 * st + 8 * a4));
+            }
+        }
+        auto load_vfrags = [&](v4i (&vf)[NST][2], int dt) __attribute__((always_inline)) {
+#pragma unroll
+            for (int st = 0; st < NST; ++st) {
+                if (DIAG && st > gw) continue;
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const uint32_t a0 = v_rd[dt] + VB + (32 * st + 16 * u) * VROW;
+                    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)INTFA_LDS(smem + a0));
+                    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)INTFA_LDS(smem + a0 + 8 * VROW));
+                    vf[st][u] = (v4i){__builtin_bit_cast(v2i, lo)[0], __builtin_bit_cast(v2i, lo)[1], __builtin_bit_cast(v2i, hi)[0], __builtin_bit_cast(v2i, hi)[1]};
+                }
+            }
+        };
+        // -------- pass 1: S^T sub-tiles, dequantise, running max
+        v16i si[NST];                                       // int8 Q K^T accumulators
+        v16f sf[NST];                                       // 16-bit Q K^T accumulators
+        auto qk_mfma = [&](int st, int ks) __attribute__((always_inline)) {
+            if (QK_INT8) si[st] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[st][ks], qreg[ks], ks ? si[st] : (v16i){0}, 0, 0, 0);
+            else sf[st] = mfma16(fr[st][ks], qreg[ks], ks ? sf[st] : (v16f){0});
+        };
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qk_mfma(0, ks);
         float t[NST][16];
         float mx = -INFINITY;
 #pragma unroll
@@ -165,75 +211,73 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
                 for (int r = 0; r < 16; ++r) t[st][r] = -INFINITY;
                 continue;
             }
-            v4i fr[KS];
+            const bool next = st + 1 < nact;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) fr[ks] = *(const v4i*)(smem + k_rd[ks] + KB + 32 * st * KROW);
-            float x[16];
-            if (QK_INT8) {
-                v16i acc = {0};
+            for (int a4 = 0; a4 < 4; ++a4) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (st + 1 < NST && next) {
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[ks], qreg[ks], acc, 0, 0, 0);
-#pragma unroll
-                for (int a4 = 0; a4 < 4; ++a4) {
-                    const v4f kk = *(const v4f*)(smem + ks_rd + SB + 4 * (32 * st + 8 * a4));
-#pragma unroll
-                    for (int b4 = 0; b4 < 4; ++b4) x[4 * a4 + b4] = (float)acc[4 * a4 + b4] * kk[b4];
+                    for (int ks = a4 * KS / 4; ks < (a4 + 1) * KS / 4; ++ks) qk_mfma(st + 1, ks);
                 }
-            } else {
-                v16f acc = {0};
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    if (IO_DT == 0) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, fr[ks]), __builtin_bit_cast(v8h, qreg[ks]), acc, 0, 0, 0);
-                    else acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fr[ks]), __builtin_bit_cast(v8bf, qreg[ks]), acc, 0, 0, 0);
+                for (int b4 = 0; b4 < 4; ++b4) {
+                    const int r = 4 * a4 + b4;
+                    float v = QK_INT8 ? (float)si[st][r] * kk[st][a4][b4] : sf[st][r];
+                    if (DIAG && st == gw && (8 * a4 + b4) > lq - 4 * lh) v = -INFINITY;
+                    t[st][r] = v;
+                    mx = fmaxf(mx, v);
                 }
-#pragma unroll
-                for (int r = 0; r < 16; ++r) x[r] = acc[r];
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float v = x[r];
-                if (DIAG && st == gw && (8 * (r >> 2) + (r & 3)) > lq - 4 * lh) v = -INFINITY;
-                t[st][r] = v;
-                mx = fmaxf(mx, v);
             }
         }
+        // V fragments of the first two d-tiles travel while the exponentials are evaluated
+        v4i vf[2][NST][2];
+        __builtin_amdgcn_sched_barrier(0);
+        load_vfrags(vf[0], 0);
+        if (1 < DT) load_vfrags(vf[1], 1);
         mx = half_pair_max(mx);
         const float m_new = fmaxf(m_run, mx * qsc);
         const float alpha = fast_exp2(m_run - m_new);
         m_run = m_new;
-        // -------- P = exp2(x*qsc - m), row sum, cast to the 16-bit type; rescale the running output
+        // -------- pass 2: P = exp2(x*qsc - m), row sum, cast to the 16-bit type
         float lsum = 0.f;
         v4i pf[NST][2];                                   // B operands: 8 x 16-bit per 16-key step
 #pragma unroll
         for (int st = 0; st < NST; ++st) {
+            if (DIAG && st > gw) continue;
+            __builtin_amdgcn_sched_barrier(0);
             float e[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) { e[r] = fast_exp2(fmaf(t[st][r], qsc, -m_new)); lsum += e[r]; }
 #pragma unroll
             for (int u = 0; u < 2; ++u)
                 pf[st][u] = IO_DT == 0 ? __builtin_bit_cast(v4i, pack_p_f16(e + 8 * u)) : __builtin_bit_cast(v4i, pack_p_bf16(e + 8 * u));
+            asm volatile("" : "+v"(lsum));
         }
         l_run = fmaf(l_run, alpha, lsum);
+        // -------- O^T[d, q] = alpha * O^T + V^T[d, key] P^T[key, q]: d-tile 0 is rescaled here, d-tile dt+1 under the
+        // MFMAs of d-tile dt
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
-        // -------- O^T[d, q] += V^T[d, key] P^T[key, q]
+        for (int r = 0; r < 16; ++r) { o_acc[0][r] *= alpha; asm volatile("" : "+v"(o_acc[0][r])); }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
-            for (int st = 0; st < NST; ++st) {
-                if (DIAG && st > gw) continue;
+            for (int a4 = 0; a4 < 4; ++a4) {
+                const int st = a4 >> 1, u = a4 & 1;
+                __builtin_amdgcn_sched_barrier(0);
+                if (!(DIAG && st > gw)) o_acc[dt] = mfma16(vf[dt & 1][st][u], pf[st][u], o_acc[dt]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (dt + 1 < DT) {
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const uint32_t a0 = v_rd[dt] + VB + (32 * st + 16 * u) * VROW;
-                    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)INTFA_LDS(smem + a0));
-                    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)INTFA_LDS(smem + a0 + 8 * VROW));
-                    const v4i a = {__builtin_bit_cast(v2i, lo)[0], __builtin_bit_cast(v2i, lo)[1], __builtin_bit_cast(v2i, hi)[0], __builtin_bit_cast(v2i, hi)[1]};
-                    if (IO_DT == 0) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, pf[st][u]), o_acc[dt], 0, 0, 0);
-                    else o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, pf[st][u]), o_acc[dt], 0, 0, 0);
+                    for (int b4 = 0; b4 < 4; ++b4) {
+                        o_acc[dt + 1][4 * a4 + b4] *= alpha;
+                        asm volatile("" : "+v"(o_acc[dt + 1][4 * a4 + b4]));
+                    }
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
+            if (dt + 2 < DT) load_vfrags(vf[dt & 1], dt + 2);
         }
     };
 
