@@ -53,7 +53,8 @@ enum {
     INTFA_ERR_ALIGN = -4,         /* pointer or row stride not 16-byte aligned */
     INTFA_ERR_DTYPE = -5,         /* unknown dtype enum */
     INTFA_ERR_WORKSPACE = -6,     /* workspace missing or too small for the requested split count */
-    INTFA_ERR_SHAPE = -7,         /* batch/heads not positive, or sizes overflow 32-bit block indices */
+    INTFA_ERR_SHAPE = -7,         /* batch/heads not positive, a row stride below head_dim, a (batch, head) slice of
+                                     k or v spanning 4 GiB or more, or sizes that overflow 32-bit block indices */
     INTFA_ERR_SPLITS = -8         /* num_splits out of range */
 };
 

@@ -24,10 +24,14 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
     if (p->io_dtype != INTFA_F16 && p->io_dtype != INTFA_BF16) return INTFA_ERR_DTYPE;
     const int64_t n_blocks = (int64_t)p->batch * p->heads * (p->seqlen / kBlockM);
     if (n_blocks * kMaxSplits >= (1ll << 31)) return INTFA_ERR_SHAPE;
+    // K and V slices are addressed through 32-bit buffer offsets: one (batch, head) slice must span less than 4 GiB
+    if ((int64_t)(p->seqlen - 1) * p->k_stride_n * qk_bytes + (int64_t)p->head_dim * qk_bytes >= (1ll << 32)) return INTFA_ERR_SHAPE;
+    if (v_bytes > 0 && (int64_t)(p->seqlen - 1) * p->v_stride_n * v_bytes + (int64_t)p->head_dim * v_bytes >= (1ll << 32)) return INTFA_ERR_SHAPE;
     if (!aligned16(p->q) || !aligned16(p->k)) return INTFA_ERR_ALIGN;
     if ((p->q_stride_n * qk_bytes) % 16 || (p->k_stride_n * qk_bytes) % 16) return INTFA_ERR_ALIGN;
     if ((p->q_stride_b * qk_bytes) % 16 || (p->q_stride_h * qk_bytes) % 16) return INTFA_ERR_ALIGN;
     if ((p->k_stride_b * qk_bytes) % 16 || (p->k_stride_h * qk_bytes) % 16) return INTFA_ERR_ALIGN;
+    if (p->k_stride_n < p->head_dim || p->q_stride_n < p->head_dim) return INTFA_ERR_SHAPE;
     KParams k{};
     k.q = (const char*)p->q; k.k = (const char*)p->k;
     k.q_sb = p->q_stride_b * qk_bytes; k.q_sh = p->q_stride_h * qk_bytes; k.q_sn = p->q_stride_n * qk_bytes;
@@ -37,6 +41,7 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
         if (!aligned16(p->v) || (reinterpret_cast<uintptr_t>(p->out) & 7u)) return INTFA_ERR_ALIGN;
         if ((p->v_stride_n * v_bytes) % 16 || (p->v_stride_b * v_bytes) % 16 || (p->v_stride_h * v_bytes) % 16) return INTFA_ERR_ALIGN;
         if ((p->o_stride_n * 2) % 8 || (p->o_stride_b * 2) % 8 || (p->o_stride_h * 2) % 8) return INTFA_ERR_ALIGN;
+        if (p->v_stride_n < p->head_dim || p->o_stride_n < p->head_dim) return INTFA_ERR_SHAPE;
         k.v = (const char*)p->v; k.out = (char*)p->out;
         k.v_sb = p->v_stride_b * v_bytes; k.v_sh = p->v_stride_h * v_bytes; k.v_sn = p->v_stride_n * v_bytes;
         k.o_sb = p->o_stride_b * 2; k.o_sh = p->o_stride_h * 2; k.o_sn = p->o_stride_n * 2;

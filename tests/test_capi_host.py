@@ -74,6 +74,8 @@ def _valid_block():
     (lambda p: setattr(p, "io_dtype", 2), -5),
     (lambda p: setattr(p, "num_splits", 4), -6),          # splits requested without a workspace
     (lambda p: setattr(p, "batch", 0), -7),
+    (lambda p: setattr(p, "q_stride_n", 64), -7),          # rows overlap: stride below head_dim
+    (lambda p: (setattr(p, "seqlen", 1 << 20), setattr(p, "k_stride_n", 1 << 13)), -7),   # a K slice of 8 GiB
     (lambda p: (setattr(p, "num_splits", 65), setattr(p, "workspace", 0x10000), setattr(p, "workspace_bytes", 1 << 40)), -8),
 ])
 def test_validation_rejects_bad_blocks_before_touching_the_gpu(mutate, code):
