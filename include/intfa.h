@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define INTFA_VERSION 1
+#define INTFA_VERSION 2
 
 /* forward variants (one entry point each, below) */
 enum { INTFA_VARIANT_FULL_INT8 = 0, INTFA_VARIANT_HALF_INT8 = 1, INTFA_VARIANT_FP16 = 2 };
@@ -60,7 +60,8 @@ enum {
 
 /*
  * Parameter block shared by the three forward variants.  Unused members of a variant are ignored
- * (q_scale/k_scale for the fp16 variant, v_scale for the half-int8 and fp16 variants).
+ * (q_scale/k_scale for the fp16 variant, v_scale for the half-int8 and fp16 variants).  k, v and their scales have
+ * heads_kv heads when that member is set.
  *
  *   variant      q, k            v               out
  *   full-int8    int8            int8            out_dtype (fp16 as in the reference, or bf16)
@@ -96,6 +97,12 @@ typedef struct intfa_fwd_params {
     int32_t num_splits;       /* <= 1: single pass; > 1: split-KV partials + combine (needs workspace) */
     void*   workspace;        /* device scratch of at least intfa_fwd_workspace_bytes() bytes, or NULL */
     size_t  workspace_bytes;
+
+    int32_t heads_kv;         /* grouped-query / multi-query attention: number of K/V heads; k, v, k_scale and v_scale
+                                 then have heads_kv heads and query head h reads K/V head h / (heads / heads_kv).
+                                 0 or heads = one K/V head per query head (the reference's Python API; its CUDA tree
+                                 has the grouped form, csrc/flash_fwd_kernel_full_qi8.h:141).  Must divide heads. */
+    int32_t reserved;         /* set to 0 */
 } intfa_fwd_params;
 
 /* Library/ABI version (INTFA_VERSION of the build). */

@@ -11,6 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libintfa.so")
 
+ABI_VERSION = 2          # INTFA_VERSION of include/intfa.h this mirror was written against
 INTFA_F16, INTFA_BF16, INTFA_F32 = 0, 1, 2
 PROUND_RNE, PROUND_REFERENCE = 0, 1
 
@@ -29,7 +30,8 @@ class FwdParams(ctypes.Structure):
             "vs_stride_b", "vs_stride_h")]
         + [(n, ctypes.c_int32) for n in ("batch", "heads", "seqlen", "head_dim", "scale_dtype", "io_dtype", "causal")]
         + [("sm_scale", ctypes.c_float), ("p_round", ctypes.c_int32), ("num_splits", ctypes.c_int32),
-           ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t)]
+           ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+           ("heads_kv", ctypes.c_int32), ("reserved", ctypes.c_int32)]
     )
 
 
@@ -74,6 +76,8 @@ def load():
     lib.intfa_quant_pertensor_workspace_bytes.argtypes = [i32, i32]
     lib.intfa_quant_pertensor.restype = ctypes.c_int
     lib.intfa_quant_pertensor.argtypes = [vp, i64, i64, i64, vp, vp, i32, i32, i32, i32, i32, vp, ctypes.c_size_t, vp]
+    if lib.intfa_version() != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH} has ABI version {lib.intfa_version()}, this package expects {ABI_VERSION}: rebuild it")
     _lib = lib
     return lib
 

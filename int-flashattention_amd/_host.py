@@ -55,8 +55,11 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
     _require_gpu(q, k, v, q_scale, k_scale, v_scale)
     d = check_head_dims(q, k, v)
     Z, H, N, _ = q.shape
-    if k.shape[:3] != q.shape[:3] or v.shape[:3] != q.shape[:3]:
-        raise ValueError("q, k and v must share [Z, H, N] (the reference passes a single N_CTX)")
+    H_kv = k.shape[1]
+    if k.shape[0] != Z or v.shape[0] != Z or k.shape[2] != N or v.shape[2] != N or v.shape[1] != H_kv:
+        raise ValueError("q, k and v must share the batch size and N (the reference passes a single N_CTX)")
+    if H % H_kv != 0:
+        raise ValueError(f"the number of query heads ({H}) must be a multiple of the number of K/V heads ({H_kv})")
     if N % BLOCK != 0:
         raise ValueError(f"sequence length {N} must be a multiple of {BLOCK} (the reference's tiles have no bounds checks either)")
     dk = max(d, MIN_HEAD_DIM)
@@ -88,6 +91,7 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
         p.vs_stride_b, p.vs_stride_h = vs.stride()
         keep.append(vs)
     p.batch, p.heads, p.seqlen, p.head_dim = Z, H, N, dk
+    p.heads_kv = H_kv
     p.io_dtype = _TORCH_TO_ENUM[out_dtype]
     p.causal = 1 if causal else 0
     p.sm_scale = float(sm_scale)

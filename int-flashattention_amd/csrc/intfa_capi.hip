@@ -18,6 +18,8 @@ int scale_size(int dt) { return dt == INTFA_F32 ? 4 : 2; }
 int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need_scales, bool need_vscale, KParams* kp) {
     if (p == nullptr || p->q == nullptr || p->k == nullptr) return INTFA_ERR_NULL;
     if (p->batch <= 0 || p->heads <= 0) return INTFA_ERR_SHAPE;
+    const int heads_kv = p->heads_kv > 0 ? p->heads_kv : p->heads;
+    if (heads_kv > p->heads || p->heads % heads_kv != 0) return INTFA_ERR_SHAPE;
     if (p->seqlen <= 0 || p->seqlen % kBlockM != 0) return INTFA_ERR_SEQLEN;
     if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256) return INTFA_ERR_HEAD_DIM;
     if (p->scale_dtype < 0 || p->scale_dtype > 2) return INTFA_ERR_DTYPE;
@@ -59,6 +61,7 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
     k.lse = p->lse;
     k.batch = p->batch; k.heads = p->heads; k.seqlen = p->seqlen; k.head_dim = p->head_dim;
     k.scale_dtype = p->scale_dtype; k.causal = p->causal ? 1 : 0;
+    k.kv_group = p->heads / heads_kv;
     k.num_splits = 1; k.blocks_per_split = p->seqlen;   // single pass: never the limit
     k.qk_scale_log2 = p->sm_scale * 1.44269504f;      // flash_atten_full_int8.py:156-157
     *kp = k;

@@ -55,6 +55,7 @@ struct KParams {
     int64_t vs_sb, vs_sh;
     int32_t batch, heads, seqlen, head_dim;
     int32_t scale_dtype, causal, num_splits, blocks_per_split;
+    int32_t kv_group;                      // query heads per K/V head (1 = every query head has its own K/V)
     int32_t pair_mblocks;                  // causal single-pass launches: one workgroup takes query blocks i and n-1-i
     float qk_scale_log2;                   // sm_scale * log2(e)
 };

@@ -58,14 +58,26 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     const int per_head = pair ? n_mblk / 2 : n_mblk * n_split;
     const int n_heads = p.batch * p.heads;
     const int bid = blockIdx.x;
+    // With grouped K/V heads (kv_group query heads share one K/V head) the unit dealt to an XCD is the K/V head: all
+    // query heads of a group run on the XCD whose L2 holds their K/V.
+    const int kv_group = p.kv_group;
+    const int per_kv = per_head * kv_group;              // workgroups per K/V head
+    const int n_kv = n_heads / kv_group;
     int head, rem;
-    if ((n_heads & 7) == 0) {                         // whole heads per XCD (see the full-int8 kernel)
-        const int xcd = bid & 7, slot = bid >> 3;
-        head = (slot / per_head) * 8 + xcd;
-        rem = slot % per_head;
-    } else {
-        head = bid / per_head;
-        rem = bid % per_head;
+    {
+        int kv_lin, r;
+        if ((n_kv & 7) == 0) {
+            const int xcd = bid & 7, slot = bid >> 3;
+            kv_lin = (slot / per_kv) * 8 + xcd;
+            r = slot % per_kv;
+        } else {
+            kv_lin = bid / per_kv;
+            r = bid % per_kv;
+        }
+        const int heads_kv = p.heads / kv_group;
+        const int bb = kv_lin / heads_kv, hk = kv_lin % heads_kv;
+        head = bb * p.heads + hk * kv_group + r / per_head;
+        rem = r % per_head;
     }
     const int mb_idx = rem / n_split;
     const int split = rem % n_split;
@@ -76,6 +88,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     int mb = mb_idx;
     if (CAUSAL) mb = (pair && job) ? mb_idx : n_mblk - 1 - mb_idx;     // heaviest query blocks first
     const int b = head / p.heads, h = head % p.heads;
+    const int hk = h / kv_group;                     // K/V head of this query head
     int nb_begin = 0, nb_end = CAUSAL ? (mb + 1) * RDIAG : (p.seqlen / BN);
     if (SPLIT) {
         nb_begin = split * p.blocks_per_split;
@@ -102,8 +115,8 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
         for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.f;
 
     // ---- global -> LDS copies
-    const char* Kg = p.k + b * p.k_sb + h * p.k_sh;
-    const char* Vg = p.v + b * p.v_sb + h * p.v_sh;
+    const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
+    const char* Vg = p.v + b * p.v_sb + hk * p.v_sh;
     const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen - 1) * p.k_sn + KROW));
     const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + VROW));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
@@ -115,7 +128,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
         issue_tile_load<VROW, SWZ_V16, BN>(v_rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane);
     };
     const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
-    const char* Ksg = QK_INT8 ? p.k_scale + (b * p.ks_sb + h * p.ks_sh) * ks_esize : nullptr;
+    const char* Ksg = QK_INT8 ? p.k_scale + (b * p.ks_sb + hk * p.ks_sh) * ks_esize : nullptr;
     const uint32_t ks_goff = (uint32_t)(tid & (BN - 1)) * (uint32_t)(p.ks_sn * ks_esize);
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
         if (!QK_INT8 || tid >= BN) return 0u;

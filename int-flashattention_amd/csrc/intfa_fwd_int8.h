@@ -53,14 +53,26 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     const int per_head = pair ? n_mblk / 2 : n_mblk * n_split;
     const int n_heads = p.batch * p.heads;
     const int bid = blockIdx.x;
+    // With grouped K/V heads (kv_group query heads share one K/V head) the unit dealt to an XCD is the K/V head: all
+    // query heads of a group run on the XCD whose L2 holds their K/V.
+    const int kv_group = p.kv_group;
+    const int per_kv = per_head * kv_group;              // workgroups per K/V head
+    const int n_kv = n_heads / kv_group;
     int head, rem;
-    if ((n_heads & 7) == 0) {
-        const int xcd = bid & 7, slot = bid >> 3;
-        head = (slot / per_head) * 8 + xcd;
-        rem = slot % per_head;
-    } else {
-        head = bid / per_head;
-        rem = bid % per_head;
+    {
+        int kv_lin, r;
+        if ((n_kv & 7) == 0) {
+            const int xcd = bid & 7, slot = bid >> 3;
+            kv_lin = (slot / per_kv) * 8 + xcd;
+            r = slot % per_kv;
+        } else {
+            kv_lin = bid / per_kv;
+            r = bid % per_kv;
+        }
+        const int heads_kv = p.heads / kv_group;
+        const int bb = kv_lin / heads_kv, hk = kv_lin % heads_kv;
+        head = bb * p.heads + hk * kv_group + r / per_head;
+        rem = r % per_head;
     }
     const int mb_idx = rem / n_split;
     const int split = rem % n_split;
@@ -71,6 +83,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     int mb = mb_idx;
     if (CAUSAL) mb = (pair && job) ? mb_idx : n_mblk - 1 - mb_idx;     // heaviest query blocks first
     const int b = head / p.heads, h = head % p.heads;
+    const int hk = h / kv_group;                     // K/V head of this query head
 
     // key-block range of this workgroup
     int nb_begin = 0, nb_end = CAUSAL ? (mb + 1) * RDIAG : (p.seqlen / BN);
@@ -99,8 +112,8 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
         for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.f;
 
     // ---- global -> LDS copies (asynchronous, straight into LDS)
-    const char* Kg = p.k + b * p.k_sb + h * p.k_sh;
-    const char* Vg = DUMP_S ? Kg : p.v + b * p.v_sb + h * p.v_sh;
+    const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
+    const char* Vg = DUMP_S ? Kg : p.v + b * p.v_sb + hk * p.v_sh;
     const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen - 1) * p.k_sn + D));
     const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + D));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
@@ -130,7 +143,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     };
     // k_scale of a block: thread t < 128 fetches the scale of key t; converted to fp32 when stored to LDS
     const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
-    const char* Ksg = p.k_scale + (b * p.ks_sb + h * p.ks_sh) * ks_esize;
+    const char* Ksg = p.k_scale + (b * p.ks_sb + hk * p.ks_sh) * ks_esize;
     const uint32_t ks_goff = (uint32_t)(tid & (BN - 1)) * (uint32_t)(p.ks_sn * ks_esize);
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {           // raw bits
         if (DUMP_S) return 0u;
@@ -408,7 +421,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     const int e_heads = pe->heads, e_seqlen = pe->seqlen;
     const int eb = head / e_heads, eh = head % e_heads;
     const float l_tot = half_pair_sum(l_run);          // in units of 1/127 when PROUND == 0
-    const float vs = load_scale(pe->v_scale, eb * pe->vs_sb + eh * pe->vs_sh, pe->scale_dtype);
+    const float vs = load_scale(pe->v_scale, eb * pe->vs_sb + (eh / pe->kv_group) * pe->vs_sh, pe->scale_dtype);
     const float out_scale = (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
     const float l_true = (PROUND == 0) ? l_tot * (1.f / 127.f) : l_tot;
     const float lse = m_run + __builtin_log2f(l_true);

@@ -25,7 +25,8 @@ def test_library_exports_every_declared_symbol():
     assert set(declared) == set(_capi.EXPORTS)
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in intfa.h but not exported by libintfa.so"
-    assert lib.intfa_version() == 1
+    header_version = int(re.search(r"#define INTFA_VERSION (\d+)", text).group(1))
+    assert lib.intfa_version() == header_version == _capi.ABI_VERSION
     assert lib.intfa_fwd_block_n(0, 128) == 128 == _host.BLOCK
     assert lib.intfa_fwd_block_n(0, 256) == 64 and lib.intfa_fwd_block_n(1, 128) == 64 and lib.intfa_fwd_block_n(2, 64) == 64
     assert lib.intfa_fwd_block_n(3, 128) < 0 and lib.intfa_fwd_block_n(0, 96) < 0
@@ -74,6 +75,7 @@ def _valid_block():
     (lambda p: setattr(p, "io_dtype", 2), -5),
     (lambda p: setattr(p, "num_splits", 4), -6),          # splits requested without a workspace
     (lambda p: setattr(p, "batch", 0), -7),
+    (lambda p: setattr(p, "heads_kv", 3), -7),             # K/V heads must divide the query heads
     (lambda p: setattr(p, "q_stride_n", 64), -7),          # rows overlap: stride below head_dim
     (lambda p: (setattr(p, "seqlen", 1 << 20), setattr(p, "k_stride_n", 1 << 13)), -7),   # a K slice of 8 GiB
     (lambda p: (setattr(p, "num_splits", 65), setattr(p, "workspace", 0x10000), setattr(p, "workspace_bytes", 1 << 40)), -8),

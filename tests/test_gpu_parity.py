@@ -275,6 +275,37 @@ def test_three_variants_order_by_precision():
     assert e_fp < e_half < e_full < 5e-2
 
 
+# ------------------------------------------------------------------------------------------ grouped K/V heads
+@pytest.mark.parametrize("variant", ["full", "half", "fp"])
+@pytest.mark.parametrize("B,H,H_kv,N,D,causal", [(1, 8, 2, 256, 128, True), (2, 16, 16 // 4, 384, 64, False), (2, 4, 1, 256, 128, True)])
+def test_grouped_kv_heads_equal_repeated_kv(variant, B, H, H_kv, N, D, causal):
+    """k, v (and their scales) with fewer heads than q: query head h reads K/V head h // (H / H_kv), i.e. the result
+    equals ordinary attention on K/V repeated along the head axis (the reference's CUDA tree has this form,
+    csrc/flash_fwd_kernel_full_qi8.h:141; its Python API does not)."""
+    g = H // H_kv
+    q, _, _, _ = O.make_inputs(B, H, N, D, seed=50)
+    _, k, v, _ = O.make_inputs(B, H_kv, N, D, seed=51)
+    q8, qs = O.quant_pertoken(q)
+    k8, ks = O.quant_pertoken(k)
+    v8, vs = O.quant_pertensor(v)
+    rep = lambda t: t.repeat_interleave(g, dim=1)
+    sm = D ** -0.5
+    if variant == "full":
+        o = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), causal, sm)
+        ref = O.attention_full_int8(q8, rep(k8), rep(v8), qs, rep(ks), rep(vs), causal, sm, block_n=M.block_n("full", D),
+                                    p_requant=O.p_requant_rne)
+        assert_same_rounding(o, ref)
+    elif variant == "half":
+        o = M.attention_int8(*gpu(q8, k8, v, qs, ks), causal, sm)
+        ref = O.attention_int8(q8, rep(k8), rep(v), qs, rep(ks), causal, sm, block_n=64)
+        assert max_abs(o, ref) <= 2e-3 and mean_rel(o, ref) <= 2e-4
+    else:
+        o = M.attention(*gpu(q, k, v), causal, sm)
+        ref = O.attention_fp(q, rep(k), rep(v), causal, sm, block_n=64)
+        assert max_abs(o, ref) <= 2e-3 and mean_rel(o, ref) <= 2e-4
+    assert o.shape == (B, H, N, D)
+
+
 # ------------------------------------------------------------------------------------------ full-size properties
 def _headline_inputs(B=4, H=32, N=4096, D=128, seed=20):
     g = torch.Generator(device=DEV).manual_seed(seed)
