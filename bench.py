@@ -41,8 +41,8 @@ WORKLOADS = {
 # HBM bytes per launch of the forward kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
 # what the same counter reads for a plain copy of known size; None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    # FETCH_SIZE 99442.4 x 1.9997 + WRITE_SIZE 131072 x 1.0 (KiB per dispatch): 194.2 MiB read + 128 MiB written
-    "full_int8_B4_H32_N4096_d128": 337848828,
+    # FETCH_SIZE x 1.9997 + WRITE_SIZE x 1.0 (KiB per dispatch, factors from a 256 MiB copy): 194.2 MiB read + 128 MiB written
+    "full_int8_B4_H32_N4096_d128": 337860823,
 }
 
 
