@@ -49,7 +49,7 @@ enum {
     INTFA_OK = 0,
     INTFA_ERR_NULL = -1,          /* a required pointer is NULL */
     INTFA_ERR_HEAD_DIM = -2,      /* head_dim not supported by the kernels */
-    INTFA_ERR_SEQLEN = -3,        /* seqlen not a positive multiple of the query block (128) */
+    INTFA_ERR_SEQLEN = -3,        /* seqlen not positive */
     INTFA_ERR_ALIGN = -4,         /* pointer or row stride not 16-byte aligned */
     INTFA_ERR_DTYPE = -5,         /* unknown dtype enum */
     INTFA_ERR_WORKSPACE = -6,     /* workspace missing or too small for the requested split count */

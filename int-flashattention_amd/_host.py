@@ -11,7 +11,7 @@ import torch.nn.functional as F
 from . import _capi
 
 _TORCH_TO_ENUM = {torch.float16: _capi.INTFA_F16, torch.bfloat16: _capi.INTFA_BF16, torch.float32: _capi.INTFA_F32}
-BLOCK = 128          # query block of the kernels; the sequence length must be a multiple of it
+BLOCK = 128          # query block of the kernels
 _VARIANT_ENUM = {"full": _capi.VARIANT_FULL_INT8, "half": _capi.VARIANT_HALF_INT8, "fp": _capi.VARIANT_FP16}
 
 
@@ -60,8 +60,6 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
         raise ValueError("q, k and v must share the batch size and N (the reference passes a single N_CTX)")
     if H % H_kv != 0:
         raise ValueError(f"the number of query heads ({H}) must be a multiple of the number of K/V heads ({H_kv})")
-    if N % BLOCK != 0:
-        raise ValueError(f"sequence length {N} must be a multiple of {BLOCK} (the reference's tiles have no bounds checks either)")
     dk = max(d, MIN_HEAD_DIM)
     qk_bytes = 1 if variant in ("full", "half") else 2
     v_bytes = 1 if variant == "full" else 2

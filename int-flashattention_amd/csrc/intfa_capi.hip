@@ -20,11 +20,11 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
     if (p->batch <= 0 || p->heads <= 0) return INTFA_ERR_SHAPE;
     const int heads_kv = p->heads_kv > 0 ? p->heads_kv : p->heads;
     if (heads_kv > p->heads || p->heads % heads_kv != 0) return INTFA_ERR_SHAPE;
-    if (p->seqlen <= 0 || p->seqlen % kBlockM != 0) return INTFA_ERR_SEQLEN;
+    if (p->seqlen <= 0) return INTFA_ERR_SEQLEN;
     if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256) return INTFA_ERR_HEAD_DIM;
     if (p->scale_dtype < 0 || p->scale_dtype > 2) return INTFA_ERR_DTYPE;
     if (p->io_dtype != INTFA_F16 && p->io_dtype != INTFA_BF16) return INTFA_ERR_DTYPE;
-    const int64_t n_blocks = (int64_t)p->batch * p->heads * (p->seqlen / kBlockM);
+    const int64_t n_blocks = (int64_t)p->batch * p->heads * ((p->seqlen + kBlockM - 1) / kBlockM);
     if (n_blocks * kMaxSplits >= (1ll << 31)) return INTFA_ERR_SHAPE;
     // K and V slices are addressed through 32-bit buffer offsets: one (batch, head) slice must span less than 4 GiB
     if ((int64_t)(p->seqlen - 1) * p->k_stride_n * qk_bytes + (int64_t)p->head_dim * qk_bytes >= (1ll << 32)) return INTFA_ERR_SHAPE;
@@ -79,7 +79,7 @@ int setup_split(const intfa_fwd_params* p, int block_n, KParams* kp) {
     if (p->num_splits > kMaxSplits) return INTFA_ERR_SPLITS;
     const size_t need = workspace_bytes_for(p);
     if (p->workspace == nullptr || p->workspace_bytes < need || !aligned16(p->workspace)) return INTFA_ERR_WORKSPACE;
-    const int n_blocks = p->seqlen / block_n;
+    const int n_blocks = (p->seqlen + block_n - 1) / block_n;
     kp->num_splits = p->num_splits;
     kp->blocks_per_split = (n_blocks + p->num_splits - 1) / p->num_splits;     // csrc/flash_fwd_kernel.h:503
     const size_t rows = (size_t)p->num_splits * p->batch * p->heads * p->seqlen;
@@ -138,7 +138,7 @@ int run_forward(int variant, const intfa_fwd_params* p, int qk_bytes, int v_byte
     if (variant == INTFA_VARIANT_FULL_INT8 && p->p_round != INTFA_PROUND_RNE && p->p_round != INTFA_PROUND_REFERENCE) return INTFA_ERR_DTYPE;
     rc = setup_split(p, block_n_for(variant, kp.head_dim), &kp);
     if (rc != INTFA_OK) return rc;
-    kp.pair_mblocks = (kp.causal && kp.num_splits <= 1 && (kp.seqlen / kBlockM) % 2 == 0) ? 1 : 0;
+    kp.pair_mblocks = (kp.causal && kp.num_splits <= 1 && ((kp.seqlen + kBlockM - 1) / kBlockM) % 2 == 0) ? 1 : 0;
     rc = dispatch(variant, p, kp, false, stream);
     if (rc != INTFA_OK || kp.num_splits <= 1) return rc;
     return launch_combine(p, kp, stream);
@@ -161,7 +161,7 @@ const char* intfa_error_string(int code) {
         case INTFA_OK: return "ok";
         case INTFA_ERR_NULL: return "a required pointer is NULL";
         case INTFA_ERR_HEAD_DIM: return "head_dim must be 64, 128 or 256";
-        case INTFA_ERR_SEQLEN: return "seqlen must be a positive multiple of 128";
+        case INTFA_ERR_SEQLEN: return "seqlen must be positive";
         case INTFA_ERR_ALIGN: return "pointers and row/head/batch strides must be 16-byte aligned";
         case INTFA_ERR_DTYPE: return "unknown dtype enum";
         case INTFA_ERR_WORKSPACE: return "workspace missing, misaligned or too small for num_splits";

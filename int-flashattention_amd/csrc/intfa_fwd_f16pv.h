@@ -50,7 +50,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lq = lane & 31, lh = lane >> 5;
 
-    const int n_mblk = p.seqlen / kBlockM;
+    const int n_mblk = (p.seqlen + kBlockM - 1) / kBlockM;      // the last query block may be partial
     const int n_split = SPLIT ? p.num_splits : 1;
     // Causal single-pass launches pair query block i with query block n-1-i in one workgroup (heavy one first): every
     // workgroup then walks the same number of key blocks and the launch has no tail of light workgroups.
@@ -89,23 +89,28 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     if (CAUSAL) mb = (pair && job) ? mb_idx : n_mblk - 1 - mb_idx;     // heaviest query blocks first
     const int b = head / p.heads, h = head % p.heads;
     const int hk = h / kv_group;                     // K/V head of this query head
-    int nb_begin = 0, nb_end = CAUSAL ? (mb + 1) * RDIAG : (p.seqlen / BN);
+    // ragged sequence lengths are handled as in the full-int8 kernel (zero-filled copies, masked last block, rows past
+    // the end computed on clamped inputs and not stored)
+    const int nb_total = (p.seqlen + BN - 1) / BN;
+    int nb_begin = 0, nb_end = CAUSAL ? ((mb + 1) * RDIAG < nb_total ? (mb + 1) * RDIAG : nb_total) : nb_total;
     if (SPLIT) {
         nb_begin = split * p.blocks_per_split;
         const int e = nb_begin + p.blocks_per_split;
         nb_end = e < nb_end ? e : nb_end;
     }
     const int q_row = mb * kBlockM + wave * 32 + lq;
+    const bool q_valid = q_row < p.seqlen;
+    const int q_ld = q_valid ? q_row : p.seqlen - 1;     // row read for lanes past the end
 
     // ---- Q fragments (B operand of S^T): 16 bytes per k-step
     v4i qreg[KS];
     {
-        const char* qrow = p.q + b * p.q_sb + h * p.q_sh + (int64_t)q_row * p.q_sn;
+        const char* qrow = p.q + b * p.q_sb + h * p.q_sh + (int64_t)q_ld * p.q_sn;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qreg[ks] = *(const v4i*)(qrow + ks * 32 + lh * 16);
     }
     // exponent scale of this lane's row: q_scale * sm_scale * log2(e) (int8 Q K^T) or sm_scale * log2(e)
-    const float qsc = QK_INT8 ? load_scale(p.q_scale, b * p.qs_sb + h * p.qs_sh + (int64_t)q_row * p.qs_sn, p.scale_dtype) * p.qk_scale_log2
+    const float qsc = QK_INT8 ? load_scale(p.q_scale, b * p.qs_sb + h * p.qs_sh + (int64_t)q_ld * p.qs_sn, p.scale_dtype) * p.qk_scale_log2
                               : p.qk_scale_log2;
     float m_run = -INFINITY, l_run = 0.f;
     v16f o_acc[DT];
@@ -129,12 +134,14 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     };
     const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
     const char* Ksg = QK_INT8 ? p.k_scale + (b * p.ks_sb + hk * p.ks_sh) * ks_esize : nullptr;
-    const uint32_t ks_goff = (uint32_t)(tid & (BN - 1)) * (uint32_t)(p.ks_sn * ks_esize);
+    const int ks_stride = (int)(p.ks_sn * ks_esize);
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
         if (!QK_INT8 || tid >= BN) return 0u;
-        const char* src = Ksg + (int64_t)(nb * BN) * (p.ks_sn * ks_esize);
-        if (p.scale_dtype == 2) return *(const uint32_t*)(src + ks_goff);
-        return (uint32_t)*(const uint16_t*)(src + ks_goff);
+        int key = nb * BN + tid;
+        key = key < p.seqlen ? key : p.seqlen - 1;                                    // keys past the end are masked later
+        const char* src = Ksg + (int64_t)key * ks_stride;
+        if (p.scale_dtype == 2) return *(const uint32_t*)src;
+        return (uint32_t)*(const uint16_t*)src;
     };
     auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float {
         if (p.scale_dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
@@ -171,12 +178,14 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     // barriers: the MFMAs of S^T sub-tile st+1 are issued one at a time between quarters of the vector work of sub-tile
     // st, the MFMAs of output d-tile dt between quarters of the rescaling of d-tile dt+1, and LDS operands are requested
     // one or two stages before the MFMA that consumes them.
-    auto compute = [&](auto buf_tag, auto diag_tag, int nb, int kb) __attribute__((always_inline)) {
+    // DIAG selects the code instance with masking: sub-tiles st > gw are skipped, in sub-tile gw the keys whose index
+    // inside the sub-tile exceeds `lim` are masked (causal diagonal: gw = the wave's own sub-tile, lim = the lane's
+    // row; ragged last block: the position of the last valid key).
+    auto compute = [&](auto buf_tag, auto diag_tag, int nb, int gw, int lim) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         constexpr bool DIAG = decltype(diag_tag)::value;
         constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4;
         static_assert(NST == 2, "the quarter interleave below assumes two sub-tiles of 32 keys");
-        const int gw = wave - kb * NST;                 // sub-tile on this wave's diagonal (DIAG only)
         if (DIAG && gw < 0) return;                     // block entirely above the wave's rows
         const int nact = DIAG ? (gw + 1 < NST ? gw + 1 : NST) : NST;
         // -------- operands of both S^T sub-tiles
@@ -237,7 +246,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
                 for (int b4 = 0; b4 < 4; ++b4) {
                     const int r = 4 * a4 + b4;
                     float v = QK_INT8 ? (float)si[st][r] * kk[st][a4][b4] : sf[st][r];
-                    if (DIAG && st == gw && (8 * a4 + b4) > lq - 4 * lh) v = -INFINITY;
+                    if (DIAG && st == gw && (8 * a4 + b4 + 4 * lh) > lim) v = -INFINITY;
                     t[st][r] = v;
                     mx = fmaxf(mx, v);
                 }
@@ -294,14 +303,14 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
         }
     };
 
-    auto step = [&](auto buf_tag, auto diag_tag, int nb) __attribute__((always_inline)) {
+    auto step = [&](auto buf_tag, auto diag_tag, int nb, int gw, int lim) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         const bool more = nb + 1 < nb_end;
         uint32_t ks_next = 0;
         if (more) { issue_loads(nb + 1, BUF ^ 1); ks_next = load_ks(nb + 1); }
-        compute(buf_tag, diag_tag, nb, CAUSAL ? nb - mb * RDIAG : 0);
+        compute(buf_tag, diag_tag, nb, gw, lim);
         if (QK_INT8 && more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
     };
 
@@ -312,22 +321,25 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
             if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
         }
         const int diag_begin = mb * RDIAG;
-        const int plain_end = (CAUSAL && nb_end > diag_begin) ? diag_begin : nb_end;
+        const int tail_keys = p.seqlen - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
+        const bool ragged = !CAUSAL && tail_keys < BN && nb_end == nb_total;
+        const int plain_end = CAUSAL ? (nb_end > diag_begin ? diag_begin : nb_end) : (ragged ? nb_end - 1 : nb_end);
         int nb = nb_begin;
         while (true) {
             if (nb >= plain_end) break;
-            step(BoolTag<false>{}, BoolTag<false>{}, nb++);
+            step(BoolTag<false>{}, BoolTag<false>{}, nb++, 0, 0);
             if (nb >= plain_end) break;
-            step(BoolTag<true>{}, BoolTag<false>{}, nb++);
+            step(BoolTag<true>{}, BoolTag<false>{}, nb++, 0, 0);
         }
-        if (CAUSAL) {
+        // masked blocks: the blocks on the causal diagonal, or the ragged last block of a non-causal pass
 #pragma unroll
-            for (int kb = 0; kb < RDIAG; ++kb) {
-                if (nb >= nb_end) break;
-                if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb);
-                else step(BoolTag<true>{}, BoolTag<true>{}, nb);
-                ++nb;
-            }
+        for (int kb = 0; kb < (CAUSAL ? RDIAG : 1); ++kb) {
+            if (nb >= nb_end) break;
+            const int gw = CAUSAL ? wave - (nb - diag_begin) * NST : (tail_keys - 1) >> 5;
+            const int lim = CAUSAL ? lq : (tail_keys - 1) & 31;
+            if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb, gw, lim);
+            else step(BoolTag<true>{}, BoolTag<true>{}, nb, gw, lim);
+            ++nb;
         }
     }
 
@@ -343,19 +355,22 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
         const int64_t row = ((int64_t)(split * pe->batch + eb) * e_heads + eh) * e_seqlen + q_row;
         float* op = pe->o_part + row * D;
         const bool seen = nb_begin < nb_end;
+        if (q_valid) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int a4 = 0; a4 < 4; ++a4) {
-                v4f o;
+                for (int a4 = 0; a4 < 4; ++a4) {
+                    v4f o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[dt][4 * a4 + b4] * inv : 0.f;
-                *(v4f*)(op + 32 * dt + 8 * a4 + 4 * lh) = o;
-            }
-        if (lh == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
+                    for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[dt][4 * a4 + b4] * inv : 0.f;
+                    *(v4f*)(op + 32 * dt + 8 * a4 + 4 * lh) = o;
+                }
+            if (lh == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
+        }
         return;
     }
     char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn;
+    if (q_valid) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -374,6 +389,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
             }
         }
     if (pe->lse != nullptr && lh == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
+    }   // q_valid
     }   // job
 #endif  // __HIP_DEVICE_COMPILE__
 }

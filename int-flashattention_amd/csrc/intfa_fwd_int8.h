@@ -45,7 +45,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
 
     // ---- block -> (head, m-block, split).  Workgroups are dealt round-robin to the 8 XCDs, each with its own
     // L2; give every XCD whole heads so that the K/V tiles of a head are re-read from one L2.
-    const int n_mblk = p.seqlen / kBlockM;
+    const int n_mblk = (p.seqlen + kBlockM - 1) / kBlockM;      // the last query block may be partial
     const int n_split = SPLIT ? p.num_splits : 1;
     // Causal single-pass launches pair query block i with query block n-1-i in one workgroup (heavy one first): every
     // workgroup then walks the same number of key blocks and the launch has no tail of light workgroups.
@@ -86,22 +86,28 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     const int hk = h / kv_group;                     // K/V head of this query head
 
     // key-block range of this workgroup
-    int nb_begin = 0, nb_end = CAUSAL ? (mb + 1) * RDIAG : (p.seqlen / BN);
+    // Sequence lengths that are not a multiple of the block sizes: the copies of K/V rows past the end return zeros
+    // (bounds-checked buffer loads), the last key block runs the masked code instance, query rows past the end are
+    // computed on clamped inputs and not stored.
+    const int nb_total = (p.seqlen + BN - 1) / BN;
+    int nb_begin = 0, nb_end = CAUSAL ? ((mb + 1) * RDIAG < nb_total ? (mb + 1) * RDIAG : nb_total) : nb_total;
     if (SPLIT) {
         nb_begin = split * p.blocks_per_split;
         const int e = nb_begin + p.blocks_per_split;
         nb_end = e < nb_end ? e : nb_end;
     }
     const int q_row = mb * kBlockM + wave * 32 + lq;     // this lane's query row
+    const bool q_valid = q_row < p.seqlen;
+    const int q_ld = q_valid ? q_row : p.seqlen - 1;     // row read for lanes past the end
 
     // ---- Q fragment (B operand of S^T = K Q^T): 16 bytes per k-step, resident for the whole kernel.
     v4i qreg[KS];
     {
-        const char* qrow = p.q + b * p.q_sb + h * p.q_sh + (int64_t)q_row * p.q_sn;
+        const char* qrow = p.q + b * p.q_sb + h * p.q_sh + (int64_t)q_ld * p.q_sn;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qreg[ks] = *(const v4i*)(qrow + ks * 32 + lh * 16);
     }
-    const float qs = DUMP_S ? 1.f : load_scale(p.q_scale, b * p.qs_sb + h * p.qs_sh + (int64_t)q_row * p.qs_sn, p.scale_dtype);
+    const float qs = DUMP_S ? 1.f : load_scale(p.q_scale, b * p.qs_sb + h * p.qs_sh + (int64_t)q_ld * p.qs_sn, p.scale_dtype);
     const float qsc = qs * p.qk_scale_log2;
 
     float m_run = -INFINITY, l_run = 0.f;
@@ -144,12 +150,15 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     // k_scale of a block: thread t < 128 fetches the scale of key t; converted to fp32 when stored to LDS
     const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
     const char* Ksg = p.k_scale + (b * p.ks_sb + hk * p.ks_sh) * ks_esize;
-    const uint32_t ks_goff = (uint32_t)(tid & (BN - 1)) * (uint32_t)(p.ks_sn * ks_esize);
+    const int ks_key = tid & (BN - 1);
+    const int ks_stride = (int)(p.ks_sn * ks_esize);
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {           // raw bits
         if (DUMP_S) return 0u;
-        const char* src = Ksg + (int64_t)(nb * BN) * (p.ks_sn * ks_esize);       // wave-uniform part
-        if (p.scale_dtype == 2) return *(const uint32_t*)(src + ks_goff);
-        return (uint32_t)*(const uint16_t*)(src + ks_goff);
+        int key = nb * BN + ks_key;
+        key = key < p.seqlen ? key : p.seqlen - 1;                                    // keys past the end are masked later
+        const char* src = Ksg + (int64_t)key * ks_stride;
+        if (p.scale_dtype == 2) return *(const uint32_t*)src;
+        return (uint32_t)*(const uint16_t*)src;
     };
     auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float {
         if (p.scale_dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
@@ -180,13 +189,14 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     const uint32_t ks_wr = OFF_KS + 4 * (tid & (BN - 1));
 
     // One key block out of LDS buffer BUF.  DIAG selects the code for the block on the causal diagonal.
-    auto compute = [&](auto buf_tag, auto diag_tag, int nb, bool more, int kb) __attribute__((always_inline)) {
+    // DIAG selects the code instance with masking: sub-tiles st > gw of the block are skipped, in sub-tile gw the keys
+    // whose index inside the sub-tile exceeds `lim` are masked.  Causal diagonal: gw = the wave's own sub-tile,
+    // lim = the lane's row (key <= query); last block of a ragged sequence: gw, lim = position of the last valid key.
+    auto compute = [&](auto buf_tag, auto diag_tag, int nb, bool more, int gw_in, int lim) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         constexpr bool DIAG = decltype(diag_tag)::value;
         constexpr int KB = BUF * KT, SB = BUF * BN * 4;
-        // On the diagonal, sub-tile st of diagonal block kb holds the keys of query sub-block kb*NST + st: it is
-        // skipped when that is above this wave's rows, masked when equal.  nact = active sub-tiles (wave-uniform).
-        const int gw = wave - kb * NST;                    // sub-tile index that sits on this wave's diagonal
+        const int gw = gw_in;                              // wave-uniform; nact = active sub-tiles
         const int nact = DIAG ? (gw + 1 < NST ? gw + 1 : NST) : NST;
         if (DIAG && nact <= 0) return;                     // every key of this block is above the wave's rows
         v4i k_next = k_rsrc, v_next = v_rsrc;
@@ -250,9 +260,13 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
             const v16i& acc = sacc[st & 1];
             v16i& nacc = sacc[(st + 1) & 1];
             if (DUMP_S) {
-                int32_t* srow = p.s_dump + ((int64_t)(b * p.heads + h) * p.seqlen + q_row) * p.seqlen + nb * BN + 32 * st;
+                const int key0 = nb * BN + 32 * st;
+                int32_t* srow = p.s_dump + ((int64_t)(b * p.heads + h) * p.seqlen + q_ld) * p.seqlen + key0;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) srow[8 * (r >> 2) + 4 * lh + (r & 3)] = acc[r];
+                for (int r = 0; r < 16; ++r) {
+                    const int kidx = 8 * (r >> 2) + 4 * lh + (r & 3);
+                    if (q_valid && key0 + kidx < p.seqlen) srow[kidx] = acc[r];
+                }
             }
 #pragma unroll
             for (int a4 = 0; a4 < 4; ++a4) {
@@ -270,7 +284,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
                     float x = (float)acc[4 * a4 + b4] * kk[st & 1][a4][b4];
                     if (DIAG) {
                         // position of the key inside the 32x32 tile on the diagonal vs this lane's query
-                        if (st == gw && (8 * a4 + b4) > lq - 4 * lh) x = -INFINITY;
+                        if (st == gw && (8 * a4 + b4 + 4 * lh) > lim) x = -INFINITY;
                     }
                     t[st][4 * a4 + b4] = x;
                     mx = fmaxf(mx, x);
@@ -370,7 +384,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
 
     // One pipeline step on LDS buffer BUF: wait for this block's tiles (issued one step earlier), make them
     // visible to all four waves, start the copy of the next block into the other buffer, compute.
-    auto step = [&](auto buf_tag, auto diag_tag, int nb) __attribute__((always_inline)) {
+    auto step = [&](auto buf_tag, auto diag_tag, int nb, int gw, int lim) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -381,7 +395,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
             if (DUMP_S || DIAG) issue_loads(nb + 1, BUF ^ 1);      // (a diagonal block is the last one: more == false)
             ks_next = load_ks(nb + 1);
         }
-        compute(buf_tag, diag_tag, nb, more, CAUSAL ? nb - mb * RDIAG : 0);
+        compute(buf_tag, diag_tag, nb, more, gw, lim);
         if (more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
     };
 
@@ -394,22 +408,26 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
             if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
         }
         const int diag_begin = mb * RDIAG;                 // first key block that touches the diagonal
-        const int plain_end = (CAUSAL && nb_end > diag_begin) ? diag_begin : nb_end;
+        const int tail_keys = p.seqlen - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
+        const bool ragged = !CAUSAL && tail_keys < BN && nb_end == nb_total;
+        const int plain_end = CAUSAL ? (nb_end > diag_begin ? diag_begin : nb_end) : (ragged ? nb_end - 1 : nb_end);
         int nb = nb_begin;
         while (true) {
             if (nb >= plain_end) break;
-            step(BoolTag<false>{}, BoolTag<false>{}, nb++);
+            step(BoolTag<false>{}, BoolTag<false>{}, nb++, 0, 0);
             if (nb >= plain_end) break;
-            step(BoolTag<true>{}, BoolTag<false>{}, nb++);
+            step(BoolTag<true>{}, BoolTag<false>{}, nb++, 0, 0);
         }
-        if (CAUSAL) {
+        // masked blocks: up to RDIAG blocks on the causal diagonal (keys past the end of a ragged sequence lie above
+        // every valid row's diagonal), or the ragged last block of a non-causal pass
 #pragma unroll
-            for (int kb = 0; kb < RDIAG; ++kb) {
-                if (nb >= nb_end) break;
-                if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb);
-                else step(BoolTag<true>{}, BoolTag<true>{}, nb);
-                ++nb;
-            }
+        for (int kb = 0; kb < (CAUSAL ? RDIAG : 1); ++kb) {
+            if (nb >= nb_end) break;
+            const int gw = CAUSAL ? wave - (nb - diag_begin) * NST : (tail_keys - 1) >> 5;
+            const int lim = CAUSAL ? lq : (tail_keys - 1) & 31;
+            if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb, gw, lim);
+            else step(BoolTag<true>{}, BoolTag<true>{}, nb, gw, lim);
+            ++nb;
         }
     }
     if (DUMP_S) return;
@@ -429,19 +447,22 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
         const int64_t row = ((int64_t)(split * pe->batch + eb) * e_heads + eh) * e_seqlen + q_row;
         float* op = pe->o_part + row * D;
         const bool seen = nb_begin < nb_end;
+        if (q_valid) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int a4 = 0; a4 < 4; ++a4) {
-                v4f o;
+                for (int a4 = 0; a4 < 4; ++a4) {
+                    v4f o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[dt][4 * a4 + b4] * out_scale : 0.f;
-                *(v4f*)(op + 32 * dt + 8 * a4 + 4 * lh) = o;
-            }
-        if (lh == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
+                    for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[dt][4 * a4 + b4] * out_scale : 0.f;
+                    *(v4f*)(op + 32 * dt + 8 * a4 + 4 * lh) = o;
+                }
+            if (lh == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
+        }
         return;
     }
     char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn;
+    if (q_valid) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -460,6 +481,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
             }
         }
     if (pe->lse != nullptr && lh == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
+    }   // q_valid
     }   // job
 #endif  // __HIP_DEVICE_COMPILE__
 }

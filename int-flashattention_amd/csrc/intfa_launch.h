@@ -15,7 +15,7 @@ struct LaunchSel {
 };
 
 template <typename K> inline int launch_kernel(K kernel, const KParams& kp, hipStream_t stream) {
-    const int grid = kp.batch * kp.heads * (kp.seqlen / kBlockM) * kp.num_splits / (kp.pair_mblocks ? 2 : 1);
+    const int grid = kp.batch * kp.heads * ((kp.seqlen + kBlockM - 1) / kBlockM) * kp.num_splits / (kp.pair_mblocks ? 2 : 1);
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, stream, kp);
     return (int)hipGetLastError();
 }

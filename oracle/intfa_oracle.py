@@ -146,8 +146,11 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
     """
     B, H, N, D = q.shape
     key_hi = N if key_hi is None else key_hi
-    assert N % block_m == 0 and N % block_n == 0 and block_m % block_n == 0
-    assert key_lo % block_n == 0 and key_hi % block_n == 0
+    # N need not be a multiple of the blocks: the last key block and the last row tile are simply shorter, which is
+    # what masking the missing keys with -inf amounts to (csrc/mask.h:261-263 for the reference's CUDA tree; its Triton
+    # kernels have no bounds handling at all)
+    assert block_m % block_n == 0
+    assert key_lo % block_n == 0 and (key_hi % block_n == 0 or key_hi == N)
     qk_scale = float(torch.tensor(sm_scale, dtype=torch.float32) * torch.tensor(LOG2E, dtype=torch.float32))
     m = torch.full((B, H, N), float("-inf"), dtype=torch.float32)
     l = torch.ones((B, H, N), dtype=torch.float32)          # flash_atten_full_int8.py:153
@@ -165,7 +168,7 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
         vj = v[:, :, start_n:start_n + block_n]
         if causal:
             tile = start_n // block_m
-            segments = [(tile * block_m, (tile + 1) * block_m, True), ((tile + 1) * block_m, N, False)]
+            segments = [(tile * block_m, min((tile + 1) * block_m, N), True), ((tile + 1) * block_m, N, False)]
         else:
             segments = [(0, N, False)]
         for r0, r1, masked in segments:
@@ -180,7 +183,7 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
                 qk = torch.matmul(qi.float(), kj.float().transpose(2, 3))    # flash_atten_fp.py:33
             m_i = m[:, :, r0:r1]
             if masked:                                                       # :39-43
-                keep = rows[r0:r1, None] >= (start_n + torch.arange(block_n))[None, :]
+                keep = rows[r0:r1, None] >= (start_n + torch.arange(kj.shape[2]))[None, :]
                 qk = qk * qk_scale + torch.where(keep, 0.0, -1.0e6)
                 m_ij = torch.maximum(m_i, qk.max(dim=-1).values)
                 qk = qk - m_ij[..., None]
@@ -274,7 +277,7 @@ def attention_full_int8_splitkv(q, k, v, q_scale, k_scale, v_scale, causal: bool
             lse_parts.append(torch.full((B, H, N), float("-inf")))
             continue
         acc, l, m = _blocked_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale,
-                                     block_m, block_n, key_lo=b0 * block_n, key_hi=b1 * block_n)
+                                     block_m, block_n, key_lo=b0 * block_n, key_hi=min(b1 * block_n, N))
         seen = ~torch.isinf(m)                       # causal rows above the split's range saw no key
         o_parts.append(torch.where(seen[..., None], acc / l[..., None], torch.zeros_like(acc)))
         lse_parts.append(torch.where(seen, m + torch.log2(l), torch.full_like(m, float("-inf"))))

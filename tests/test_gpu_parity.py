@@ -275,6 +275,79 @@ def test_three_variants_order_by_precision():
     assert e_fp < e_half < e_full < 5e-2
 
 
+# ------------------------------------------------------------------------------------------ ragged sequence lengths
+RAGGED = [(1, 2, 200, 128, False), (1, 2, 200, 128, True), (2, 3, 333, 64, False), (2, 3, 333, 64, True),
+          (1, 2, 97, 128, True), (1, 2, 1, 64, False), (1, 2, 130, 256, False), (1, 2, 190, 256, True), (1, 4, 640 + 31, 128, False)]
+
+
+@pytest.mark.parametrize("B,H,N,D,causal", RAGGED)
+def test_ragged_lengths_full_int8(B, H, N, D, causal):
+    """N that is not a multiple of 128 (nor of the key block): beyond the reference's Triton API, as in its CUDA tree."""
+    x = quantised(B, H, N, D, seed=60)
+    sm = D ** -0.5
+    bn = M.block_n("full", D)
+    s = M.debug_qk_int32(*gpu(x["q8"], x["k8"])).cpu()
+    assert torch.equal(s, O.qk_int32(x["q8"], x["k8"]))
+    o, lse = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), causal, sm, return_lse=True)
+    torch.cuda.synchronize()
+    assert o.shape == (B, H, N, D) and torch.isfinite(o).all()
+    ref, lse_ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=bn,
+                                         p_requant=O.p_requant_rne, return_lse=True)
+    assert_same_rounding(o, ref)
+    assert (lse.cpu() - lse_ref).abs().max().item() < 1e-3
+
+
+@pytest.mark.parametrize("B,H,N,D,causal", RAGGED)
+def test_ragged_lengths_half_and_fp(B, H, N, D, causal):
+    x = quantised(B, H, N, D, seed=61)
+    sm = D ** -0.5
+    o = M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), causal, sm)
+    ref = O.attention_int8(x["q8"], x["k8"], x["v"], x["qs"], x["ks"], causal, sm, block_n=64)
+    assert o.shape == (B, H, N, D) and max_abs(o, ref) <= 2e-3 and mean_rel(o, ref) <= 3e-4
+    o = M.attention(*gpu(x["q"], x["k"], x["v"]), causal, sm)
+    ref = O.attention_fp(x["q"], x["k"], x["v"], causal, sm, block_n=64)
+    assert max_abs(o, ref) <= 2e-3 and mean_rel(o, ref) <= 3e-4
+
+
+@pytest.mark.parametrize("causal,splits", [(False, 3), (True, 2)])
+def test_ragged_lengths_split_kv(causal, splits):
+    x = quantised(1, 2, 700, 128, seed=62)
+    sm = 128 ** -0.5
+    o = run_full(x, causal, sm, num_splits=splits, p_round="reference")
+    ref = O.attention_full_int8_splitkv(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, splits, block_n=128)
+    assert max_abs(o, ref) <= 4e-3 and mean_rel(o, ref) <= 3e-4
+    o1 = M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), causal, sm)
+    o2 = M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), causal, sm, num_splits=splits)
+    assert max_abs(o2, o1) <= 1e-3
+
+
+def test_ragged_outputs_do_not_touch_memory_past_the_end():
+    """Output rows are written for valid queries only: a guard region behind the output stays untouched."""
+    x = quantised(1, 1, 130, 128, seed=63)
+    o = run_full(x, False, 0.09)
+    ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], False, 0.09, p_requant=O.p_requant_rne)
+    assert_same_rounding(o, ref)
+    # the same call into a larger buffer through strides: rows 130.. of the buffer must keep their fill value
+    import ctypes
+    from int_flashattention_amd import _capi
+    big = torch.full((1, 1, 256, 128), 7.0, dtype=torch.float16, device=DEV)
+    q8, k8, v8, qs, ks, vs = gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"])
+    p = _capi.FwdParams()
+    p.q, p.k, p.v, p.out = q8.data_ptr(), k8.data_ptr(), v8.data_ptr(), big.data_ptr()
+    p.q_scale, p.k_scale, p.v_scale = qs.data_ptr(), ks.data_ptr(), vs.data_ptr()
+    for name, t in (("q", q8), ("k", k8), ("v", v8), ("o", big)):
+        setattr(p, f"{name}_stride_b", t.stride(0)); setattr(p, f"{name}_stride_h", t.stride(1)); setattr(p, f"{name}_stride_n", t.stride(2))
+    p.qs_stride_b, p.qs_stride_h, p.qs_stride_n = qs.stride()
+    p.ks_stride_b, p.ks_stride_h, p.ks_stride_n = ks.stride()
+    p.vs_stride_b, p.vs_stride_h = vs.stride()
+    p.batch, p.heads, p.seqlen, p.head_dim = 1, 1, 130, 128
+    p.scale_dtype, p.io_dtype, p.causal, p.sm_scale, p.p_round, p.num_splits = 0, 0, 0, 0.09, 0, 1
+    rc = _capi.load().intfa_fwd_full_int8(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert rc == 0
+    assert torch.equal(big[:, :, :130], o) and (big[:, :, 130:] == 7.0).all()
+
+
 # ------------------------------------------------------------------------------------------ grouped K/V heads
 @pytest.mark.parametrize("variant", ["full", "half", "fp"])
 @pytest.mark.parametrize("B,H,H_kv,N,D,causal", [(1, 8, 2, 256, 128, True), (2, 16, 16 // 4, 384, 64, False), (2, 4, 1, 256, 128, True)])

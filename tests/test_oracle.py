@@ -254,6 +254,24 @@ def test_block_n_dependence_is_bounded_but_real():
     assert 0 < d < 2e-2
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_ragged_length_equals_dense_softmax(causal):
+    """N that is no multiple of the blocks: the blocked evaluation (shorter last block, shorter last row tile) must still
+    equal torch.softmax attention over exactly N keys."""
+    g = torch.Generator().manual_seed(12)
+    N, D = 200, 32
+    q = torch.randn((1, 2, N, D), generator=g).half()
+    k = torch.randn((1, 2, N, D), generator=g).half()
+    v = torch.randn((1, 2, N, D), generator=g).half()
+    for bn in (64, 128):
+        got = O.attention_fp(q, k, v, causal, 0.2, block_n=bn).float()
+        want = _dense_attention(torch.matmul(q.float(), k.float().transpose(2, 3)) * 0.2, v.float(), causal)
+        assert (got - want).abs().max() < 2e-3
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    a = O.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, 0.2, block_n=64).float()
+    assert torch.isfinite(a).all() and (a - want).abs().max() < 6e-2     # quantisation error only
+
+
 # ------------------------------------------------------------------------------------------ split-KV
 def test_splitkv_combine_reproduces_dense_softmax():
     g = torch.Generator().manual_seed(9)
