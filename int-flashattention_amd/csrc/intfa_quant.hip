@@ -25,14 +25,25 @@ template <int DT> __device__ __forceinline__ uint16_t from_f32(float f) {      /
 // |x| of a 16-bit float as an unsigned integer: monotonic in |x| for finite values, so max works on the bits
 __device__ __forceinline__ uint32_t abs_bits(uint16_t b) { return b & 0x7fffu; }
 
+// A row's divisor is fixed, so the correctly rounded quotient x / scale is formed from the correctly rounded reciprocal
+// (one IEEE division per lane and row) with one multiply and two fused multiply-adds per element:
+//     q0 = RN(x * r),  e = x - q0 * scale (exact in one fma),  q = RN(q0 + e * r) = RN(x / scale)
+// (Markstein's correction step; it needs r = RN(1 / scale), which the IEEE division delivers, and a divisor whose
+// significand is not all ones, which a 16-bit scale cannot be).
+struct RowDivisor { float scale, recip; };
+__device__ __forceinline__ RowDivisor make_divisor(float scale) { return {scale, 1.0f / scale}; }
+
 // round(x / scale) truncated to int8, both operands and the quotient in the 16-bit type
-template <int DT> __device__ __forceinline__ int quant_one(uint16_t xb, float scale) {
-    const float q16 = to_f32<DT>(from_f32<DT>(to_f32<DT>(xb) / scale));
-    const float r = __builtin_rintf(q16);
-    return (r == r) ? (int)r : 0;                                               // NaN (zero row) -> 0
+template <int DT> __device__ __forceinline__ int quant_one(uint16_t xb, RowDivisor d) {
+    const float x = to_f32<DT>(xb);
+    const float q0 = x * d.recip;
+    const float e = __builtin_fmaf(-q0, d.scale, x);
+    const float q = __builtin_fmaf(e, d.recip, q0);
+    const float r = __builtin_rintf(to_f32<DT>(from_f32<DT>(q)));
+    return (__builtin_fabsf(r) < 2147483648.0f) ? (int)r : 0;                   // NaN / infinity (zero scale) -> 0
 }
 
-template <int DT> __device__ __forceinline__ void quant_store8(const v4i raw, float scale, char* dst) {
+template <int DT> __device__ __forceinline__ void quant_store8(const v4i raw, RowDivisor scale, char* dst) {
     int out[2];
 #pragma unroll
     for (int w = 0; w < 2; ++w) {
@@ -103,7 +114,7 @@ template <int DT, int LPR> __global__ void __launch_bounds__(256) quant_pertoken
             if (row >= rows) continue;
             const uint16_t sbits = from_f32<DT>(to_f32<DT>((uint16_t)m) / 127.0f);
             if (sub == 0) ((uint16_t*)p.scale)[row] = sbits;
-            quant_store8<DT>(raw[u], to_f32<DT>(sbits), p.q8 + (int64_t)row * p.head_dim + sub * 8);
+            quant_store8<DT>(raw[u], make_divisor(to_f32<DT>(sbits)), p.q8 + (int64_t)row * p.head_dim + sub * 8);
         }
     }
 }
@@ -162,7 +173,7 @@ template <int DT, int LPR> __global__ void __launch_bounds__(256) quant_slice_ap
             if (row >= rows) continue;
             const uint16_t sbits = from_f32<DT>(to_f32<DT>((uint16_t)p.amax[bh[u]]) / 127.0f);
             if (row == bh[u] * (uint32_t)p.seqlen && sub == 0) ((uint16_t*)p.scale)[bh[u]] = sbits;
-            quant_store8<DT>(raw[u], to_f32<DT>(sbits), p.q8 + (int64_t)row * p.head_dim + sub * 8);
+            quant_store8<DT>(raw[u], make_divisor(to_f32<DT>(sbits)), p.q8 + (int64_t)row * p.head_dim + sub * 8);
         }
     }
 }

@@ -79,3 +79,27 @@ def test_quantisers_full_size_properties():
     assert torch.equal(q[b:b + 1, h:h + 1].cpu(), q_r) and torch.equal(s[b:b + 1, h:h + 1].cpu(), s_r)
     q_r, s_r = O.quant_pertensor(x[b:b + 1, h:h + 1].cpu())
     assert torch.equal(qv[b:b + 1, h:h + 1].cpu(), q_r) and torch.equal(sv[b:b + 1, h:h + 1].cpu(), s_r)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_quantisers_every_16bit_value_against_many_scales(dtype):
+    """Every finite value of the 16-bit type divided by 96 different row scales: the kernels form the quotient from a
+    reciprocal with a correction step, which must round exactly like the oracle's division."""
+    bits = torch.arange(0, 1 << 16, dtype=torch.int32)
+    allv = bits.to(torch.int16).view(dtype)
+    allv = allv[torch.isfinite(allv.float())]
+    g = torch.Generator().manual_seed(99)
+    maxima = torch.cat([torch.tensor([127.0, 1.0, 0.33, 6.0e-5, 60000.0, 3.0, 2.0 ** -10, 1.5, 0.999, 254.0]),
+                        torch.rand(86, generator=g) * 8 + 0.01]).to(dtype)
+    rows = []
+    for m in maxima:
+        vals = allv[allv.float().abs() <= m.float().abs()]
+        pad = (-vals.numel()) % 15
+        vals = torch.cat([vals, vals[:pad]])
+        block = torch.cat([m.expand(vals.numel() // 15, 1), vals.view(-1, 15)], dim=1)      # the maximum leads every row
+        rows.append(block)
+    x = torch.cat(rows)[None, None].contiguous()                                           # [1, 1, R, 16]
+    q_t, s_t = M.quant_pertoken(x.to(DEV))
+    q_r, s_r = O.quant_pertoken(x)
+    assert torch.equal(s_t.cpu(), s_r)
+    assert torch.equal(q_t.cpu(), q_r)
