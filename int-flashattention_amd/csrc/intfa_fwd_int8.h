@@ -19,24 +19,36 @@ namespace intfa {
 template <bool V> struct BoolTag { static constexpr bool value = V; };
 
 // Key block length of the full-int8 kernel: 128 keys, or 64 at head_dim 256 (registers and LDS).
-template <int D> struct FullInt8Geom { static constexpr int NST = D <= 128 ? 4 : 2; static constexpr int BN = 32 * NST; };
+template <int D> struct FullInt8Geom {
+    static constexpr int NST = D <= 128 ? 4 : 2;
+    static constexpr int BN = 32 * NST;
+    // Output columns one workgroup produces.  At head_dim 256 the 128 fp32 output registers per lane of a full-width
+    // workgroup would leave room for one wave per SIMD only, so the columns are split over two workgroups that each
+    // redo Q K^T and the softmax and multiply P with their half of V: two waves per SIMD fit again.
+    static constexpr int DV = D <= 128 ? D : 128;
+    static constexpr int NHALF = D / DV;
+};
 
 template <int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUMP_S, bool SPLIT>
-__global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_kernel(const KParams p) {
+__global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T (32 bytes of head_dim each)
-    constexpr int DT = D / 32;                   // 32-wide output tiles along head_dim
+    constexpr int DV = DUMP_S ? D : FullInt8Geom<D>::DV;       // output columns of this workgroup
+    constexpr int NHALF = D / DV;                // workgroups that share one query block (column halves)
+    constexpr int DT = DV / 32;                  // 32-wide output tiles along head_dim
     constexpr int NST = FullInt8Geom<D>::NST;    // 32-key sub-tiles per key block
     constexpr int BN = FullInt8Geom<D>::BN;      // keys per block
     constexpr int RDIAG = kBlockM / BN;          // key blocks that overlap the causal diagonal of a query block
-    constexpr int KT = BN * D;                   // bytes of one K tile (and of one int8 V tile)
-    constexpr int CH = D / 16;                   // 16-byte chunks per row
-    constexpr int SWM = (CH < 8 ? CH : 8) - 1;   // swizzle mask
+    constexpr int KT = BN * D;                   // bytes of one K tile
+    constexpr int VT = BN * DV;                  // bytes of one int8 V tile (this workgroup's columns)
+    constexpr int CH = D / 16;                   // 16-byte chunks per K row
+    constexpr int CHV = DV / 16;                 // 16-byte chunks per V row
+    constexpr int SWM = (CHV < 8 ? CHV : 8) - 1; // swizzle mask of V rows
     // LDS map (bytes)
     constexpr int OFF_KS = 0;                    // two fp32 k_scale vectors
     constexpr int OFF_K = 2 * BN * 4;            // two K tiles
     constexpr int OFF_V = OFF_K + 2 * KT;        // two V tiles
-    constexpr int LDS_BYTES = OFF_V + 2 * KT;
+    constexpr int LDS_BYTES = OFF_V + 2 * VT;
     __shared__ __attribute__((aligned(1024))) char smem[LDS_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -50,7 +62,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     // Causal single-pass launches pair query block i with query block n-1-i in one workgroup (heavy one first): every
     // workgroup then walks the same number of key blocks and the launch has no tail of light workgroups.
     const bool pair = CAUSAL && !SPLIT && p.pair_mblocks != 0;
-    const int per_head = pair ? n_mblk / 2 : n_mblk * n_split;
+    const int per_head = (pair ? n_mblk / 2 : n_mblk * n_split) * NHALF;
     const int n_heads = p.batch * p.heads;
     const int bid = blockIdx.x;
     // With grouped K/V heads (kv_group query heads share one K/V head) the unit dealt to an XCD is the K/V head: all
@@ -74,8 +86,9 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
         head = bb * p.heads + hk * kv_group + r / per_head;
         rem = r % per_head;
     }
-    const int mb_idx = rem / n_split;
-    const int split = rem % n_split;
+    const int half = rem % NHALF;                // column half of this workgroup (0 when the columns are not split)
+    const int mb_idx = (rem / NHALF) / n_split;
+    const int split = (rem / NHALF) % n_split;
     const int njobs = pair ? 2 : 1;
 #pragma clang loop unroll(disable)
     for (int job = 0; job < njobs; ++job) {
@@ -119,20 +132,21 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
 
     // ---- global -> LDS copies (asynchronous, straight into LDS)
     const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
-    const char* Vg = DUMP_S ? Kg : p.v + b * p.v_sb + hk * p.v_sh;
+    const char* Vg = DUMP_S ? Kg : p.v + b * p.v_sb + hk * p.v_sh + half * DV;
     const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen - 1) * p.k_sn + D));
-    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + D));
+    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + DV));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
     const auto k_lane = tile_load_lane<D, SWZ_K, BN>(k_sn, wave, lane);
-    const auto v_lane = tile_load_lane<D, SWZ_V8, BN>(v_sn, wave, lane);
+    const auto v_lane = tile_load_lane<DV, SWZ_V8, BN>(v_sn, wave, lane);
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
     auto issue_loads = [&](int nb, int buf) __attribute__((always_inline)) {
         issue_tile_load<D, SWZ_K, BN>(k_rsrc, (uint32_t)(nb * BN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane);
-        if (!DUMP_S) issue_tile_load<D, SWZ_V8, BN>(v_rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * KT, wave, v_lane);
+        if (!DUMP_S) issue_tile_load<DV, SWZ_V8, BN>(v_rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane);
     };
     // The copy of the NEXT block is issued in slices spread over the stages of the current block (one K slice per
     // S^T sub-tile stage, one V slice per output d-tile stage) so that the waves do not queue behind a burst.
     constexpr int DMA_PARTS = TileLoadLane<D, SWZ_K, BN>::NINST / 4;
+    constexpr int V_PARTS = TileLoadLane<DV, SWZ_V8, BN>::NINST / 4;
     // When there is no next block the slices are issued against an empty resource (num_records = 0: every access
     // is out of range and touches no memory), which keeps the stages free of branches.
     auto issue_k_slice = [&](v4i rsrc, int nb, int buf, int stage, int nstages) __attribute__((always_inline)) {
@@ -143,9 +157,9 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     };
     auto issue_v_slice = [&](v4i rsrc, int nb, int buf, int stage, int nstages) __attribute__((always_inline)) {
 #pragma unroll
-        for (int it = 0; it < DMA_PARTS; ++it)
-            if (it * nstages / DMA_PARTS == stage)
-                issue_tile_part<D, SWZ_V8, BN>(rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * KT, wave, v_lane, it);
+        for (int it = 0; it < V_PARTS; ++it)
+            if (it * nstages / V_PARTS == stage)
+                issue_tile_part<DV, SWZ_V8, BN>(rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane, it);
     };
     // k_scale of a block: thread t < 128 fetches the scale of key t; converted to fp32 when stored to LDS
     const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
@@ -178,12 +192,12 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     // key row 8*(j>>2) + 4*lh + (j&3), j = s/2 (+16 for the second load, +32 per sub-tile), 8-byte half s&1
     const int g16 = lane >> 4, i16 = lane & 15, jj = i16 >> 1;
     const int v_row0 = 8 * (jj >> 2) + 4 * lh + (jj & 3);
-    const int v_swz = swz_v8<D>(v_row0) & SWM;
+    const int v_swz = swz_v8<DV>(v_row0) & SWM;
     uint32_t v_rd[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
         const int c = 2 * dt + (g16 & 1);
-        v_rd[dt] = OFF_V + v_row0 * D + 8 * (i16 & 1) + (((c & SWM) ^ v_swz) << 4) + ((c & ~SWM) << 4);
+        v_rd[dt] = OFF_V + v_row0 * DV + 8 * (i16 & 1) + (((c & SWM) ^ v_swz) << 4) + ((c & ~SWM) << 4);
     }
     const uint32_t ks_rd = OFF_KS + 16 * lh;     // + 4 * (32*st + 8*a4) per read
     const uint32_t ks_wr = OFF_KS + 4 * (tid & (BN - 1));
@@ -195,7 +209,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     auto compute = [&](auto buf_tag, auto diag_tag, int nb, bool more, int gw_in, int lim) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         constexpr bool DIAG = decltype(diag_tag)::value;
-        constexpr int KB = BUF * KT, SB = BUF * BN * 4;
+        constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4;
         const int gw = gw_in;                              // wave-uniform; nact = active sub-tiles
         const int nact = DIAG ? (gw + 1 < NST ? gw + 1 : NST) : NST;
         if (DIAG && nact <= 0) return;                     // every key of this block is above the wave's rows
@@ -213,9 +227,9 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
             for (int st = 0; st < NST; ++st) {
                 if (DIAG && st > gw) continue;
                 const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                    (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[dt] + KB + (32 * st) * D));
+                    (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[dt] + VB + (32 * st) * DV));
                 const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                    (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[dt] + KB + (32 * st + 16) * D));
+                    (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[dt] + VB + (32 * st + 16) * DV));
                 vf[st] = (v4i){lo[0], lo[1], hi[0], hi[1]};
             }
         };
@@ -445,7 +459,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
     const float lse = m_run + __builtin_log2f(l_true);
     if (SPLIT) {
         const int64_t row = ((int64_t)(split * pe->batch + eb) * e_heads + eh) * e_seqlen + q_row;
-        float* op = pe->o_part + row * D;
+        float* op = pe->o_part + row * D + half * DV;
         const bool seen = nb_begin < nb_end;
         if (q_valid) {
 #pragma unroll
@@ -457,11 +471,11 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
                     for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[dt][4 * a4 + b4] * out_scale : 0.f;
                     *(v4f*)(op + 32 * dt + 8 * a4 + 4 * lh) = o;
                 }
-            if (lh == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
+            if (lh == 0 && half == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
         }
         return;
     }
-    char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn;
+    char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn + half * DV * 2;
     if (q_valid) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -480,7 +494,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_full_int8_ke
                 *(v4s*)(orow + d0 * 2) = o;
             }
         }
-    if (pe->lse != nullptr && lh == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
+    if (pe->lse != nullptr && lh == 0 && half == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
     }   // q_valid
     }   // job
 #endif  // __HIP_DEVICE_COMPILE__
