@@ -49,7 +49,7 @@ enum {
     INTFA_OK = 0,
     INTFA_ERR_NULL = -1,          /* a required pointer is NULL */
     INTFA_ERR_HEAD_DIM = -2,      /* head_dim not supported by the kernels */
-    INTFA_ERR_SEQLEN = -3,        /* seqlen not positive */
+    INTFA_ERR_SEQLEN = -3,        /* seqlen not positive, or causal with seqlen_k != seqlen */
     INTFA_ERR_ALIGN = -4,         /* pointer or row stride not 16-byte aligned */
     INTFA_ERR_DTYPE = -5,         /* unknown dtype enum */
     INTFA_ERR_WORKSPACE = -6,     /* workspace missing or too small for the requested split count */
@@ -102,7 +102,9 @@ typedef struct intfa_fwd_params {
                                  then have heads_kv heads and query head h reads K/V head h / (heads / heads_kv).
                                  0 or heads = one K/V head per query head (the reference's Python API; its CUDA tree
                                  has the grouped form, csrc/flash_fwd_kernel_full_qi8.h:141).  Must divide heads. */
-    int32_t reserved;         /* set to 0 */
+    int32_t seqlen_k;         /* number of keys when it differs from the number of queries (cross attention, decoding
+                                 against a cache): k, v and k_scale then have seqlen_k rows.  0 = seqlen.  Not with
+                                 causal (the reference's mask is defined for equal lengths). */
 } intfa_fwd_params;
 
 /* Library/ABI version (INTFA_VERSION of the build). */
@@ -136,7 +138,8 @@ int intfa_fwd_fp16(const intfa_fwd_params* p, void* stream);
 
 /* Debug export of the int32 accumulators S = Q8 K8^T produced by the same MFMA tile code the forward
  * uses (flash_atten_full_int8.py:36).  s_out is [batch, heads, seqlen, seqlen] int32, contiguous.
- * Uses q, k and their strides, batch, heads, seqlen, head_dim of the block. */
+ * s_out is [batch, heads, seqlen, seqlen_k].  Uses q, k and their strides, batch, heads, seqlen, seqlen_k, head_dim
+ * of the block. */
 int intfa_debug_qk_int32(const intfa_fwd_params* p, int32_t* s_out, void* stream);
 
 /* quant_pertoken(X) -> (int8 X, scale) of the reference's harness (benchmark.py:96-100): per row of head_dim

@@ -31,7 +31,7 @@ class FwdParams(ctypes.Structure):
         + [(n, ctypes.c_int32) for n in ("batch", "heads", "seqlen", "head_dim", "scale_dtype", "io_dtype", "causal")]
         + [("sm_scale", ctypes.c_float), ("p_round", ctypes.c_int32), ("num_splits", ctypes.c_int32),
            ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
-           ("heads_kv", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+           ("heads_kv", ctypes.c_int32), ("seqlen_k", ctypes.c_int32)]
     )
 
 

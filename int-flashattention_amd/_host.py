@@ -56,8 +56,11 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
     d = check_head_dims(q, k, v)
     Z, H, N, _ = q.shape
     H_kv = k.shape[1]
-    if k.shape[0] != Z or v.shape[0] != Z or k.shape[2] != N or v.shape[2] != N or v.shape[1] != H_kv:
-        raise ValueError("q, k and v must share the batch size and N (the reference passes a single N_CTX)")
+    N_k = k.shape[2]
+    if k.shape[0] != Z or v.shape[0] != Z or v.shape[2] != N_k or v.shape[1] != H_kv:
+        raise ValueError("q, k and v must share the batch size, and k and v their heads and length")
+    if causal and N_k != N:
+        raise ValueError("causal attention needs as many keys as queries (the reference passes a single N_CTX)")
     if H % H_kv != 0:
         raise ValueError(f"the number of query heads ({H}) must be a multiple of the number of K/V heads ({H_kv})")
     dk = max(d, MIN_HEAD_DIM)
@@ -90,6 +93,7 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
         keep.append(vs)
     p.batch, p.heads, p.seqlen, p.head_dim = Z, H, N, dk
     p.heads_kv = H_kv
+    p.seqlen_k = N_k
     p.io_dtype = _TORCH_TO_ENUM[out_dtype]
     p.causal = 1 if causal else 0
     p.sm_scale = float(sm_scale)
@@ -118,12 +122,14 @@ def debug_qk_int32(q8: torch.Tensor, k8: torch.Tensor) -> torch.Tensor:
     Z, H, N, d = q8.shape
     dk = max(d, MIN_HEAD_DIM)
     q_, k_ = _rowmajor(_pad_head_dim(q8, dk), 1), _rowmajor(_pad_head_dim(k8, dk), 1)
-    s = torch.empty((Z, H, N, N), dtype=torch.int32, device=q8.device)
+    N_k = k8.shape[2]
+    s = torch.empty((Z, H, N, N_k), dtype=torch.int32, device=q8.device)
     p = _capi.FwdParams()
     p.q, p.k = q_.data_ptr(), k_.data_ptr()
     p.q_stride_b, p.q_stride_h, p.q_stride_n = q_.stride()[:3]
     p.k_stride_b, p.k_stride_h, p.k_stride_n = k_.stride()[:3]
     p.batch, p.heads, p.seqlen, p.head_dim = Z, H, N, dk
+    p.seqlen_k = N_k
     p.scale_dtype, p.io_dtype = _capi.INTFA_F32, _capi.INTFA_F16
     stream = torch.cuda.current_stream(q8.device).cuda_stream
     with torch.cuda.device(q8.device):

@@ -20,15 +20,17 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
     if (p->batch <= 0 || p->heads <= 0) return INTFA_ERR_SHAPE;
     const int heads_kv = p->heads_kv > 0 ? p->heads_kv : p->heads;
     if (heads_kv > p->heads || p->heads % heads_kv != 0) return INTFA_ERR_SHAPE;
-    if (p->seqlen <= 0) return INTFA_ERR_SEQLEN;
+    if (p->seqlen <= 0 || p->seqlen_k < 0) return INTFA_ERR_SEQLEN;
+    const int seqlen_k = p->seqlen_k > 0 ? p->seqlen_k : p->seqlen;
+    if (p->causal && seqlen_k != p->seqlen) return INTFA_ERR_SEQLEN;      // the causal mask is defined for equal lengths
     if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256) return INTFA_ERR_HEAD_DIM;
     if (p->scale_dtype < 0 || p->scale_dtype > 2) return INTFA_ERR_DTYPE;
     if (p->io_dtype != INTFA_F16 && p->io_dtype != INTFA_BF16) return INTFA_ERR_DTYPE;
     const int64_t n_blocks = (int64_t)p->batch * p->heads * ((p->seqlen + kBlockM - 1) / kBlockM);
     if (n_blocks * kMaxSplits >= (1ll << 31)) return INTFA_ERR_SHAPE;
     // K and V slices are addressed through 32-bit buffer offsets: one (batch, head) slice must span less than 4 GiB
-    if ((int64_t)(p->seqlen - 1) * p->k_stride_n * qk_bytes + (int64_t)p->head_dim * qk_bytes >= (1ll << 32)) return INTFA_ERR_SHAPE;
-    if (v_bytes > 0 && (int64_t)(p->seqlen - 1) * p->v_stride_n * v_bytes + (int64_t)p->head_dim * v_bytes >= (1ll << 32)) return INTFA_ERR_SHAPE;
+    if ((int64_t)(seqlen_k - 1) * p->k_stride_n * qk_bytes + (int64_t)p->head_dim * qk_bytes >= (1ll << 32)) return INTFA_ERR_SHAPE;
+    if (v_bytes > 0 && (int64_t)(seqlen_k - 1) * p->v_stride_n * v_bytes + (int64_t)p->head_dim * v_bytes >= (1ll << 32)) return INTFA_ERR_SHAPE;
     if (!aligned16(p->q) || !aligned16(p->k)) return INTFA_ERR_ALIGN;
     if ((p->q_stride_n * qk_bytes) % 16 || (p->k_stride_n * qk_bytes) % 16) return INTFA_ERR_ALIGN;
     if ((p->q_stride_b * qk_bytes) % 16 || (p->q_stride_h * qk_bytes) % 16) return INTFA_ERR_ALIGN;
@@ -59,7 +61,7 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
         k.v_scale = (const char*)p->v_scale; k.vs_sb = p->vs_stride_b; k.vs_sh = p->vs_stride_h;
     }
     k.lse = p->lse;
-    k.batch = p->batch; k.heads = p->heads; k.seqlen = p->seqlen; k.head_dim = p->head_dim;
+    k.batch = p->batch; k.heads = p->heads; k.seqlen = p->seqlen; k.seqlen_k = seqlen_k; k.head_dim = p->head_dim;
     k.scale_dtype = p->scale_dtype; k.causal = p->causal ? 1 : 0;
     k.kv_group = p->heads / heads_kv;
     k.num_splits = 1; k.blocks_per_split = p->seqlen;   // single pass: never the limit
@@ -79,7 +81,7 @@ int setup_split(const intfa_fwd_params* p, int block_n, KParams* kp) {
     if (p->num_splits > kMaxSplits) return INTFA_ERR_SPLITS;
     const size_t need = workspace_bytes_for(p);
     if (p->workspace == nullptr || p->workspace_bytes < need || !aligned16(p->workspace)) return INTFA_ERR_WORKSPACE;
-    const int n_blocks = (p->seqlen + block_n - 1) / block_n;
+    const int n_blocks = ((p->seqlen_k > 0 ? p->seqlen_k : p->seqlen) + block_n - 1) / block_n;
     kp->num_splits = p->num_splits;
     kp->blocks_per_split = (n_blocks + p->num_splits - 1) / p->num_splits;     // csrc/flash_fwd_kernel.h:503
     const size_t rows = (size_t)p->num_splits * p->batch * p->heads * p->seqlen;
@@ -161,7 +163,7 @@ const char* intfa_error_string(int code) {
         case INTFA_OK: return "ok";
         case INTFA_ERR_NULL: return "a required pointer is NULL";
         case INTFA_ERR_HEAD_DIM: return "head_dim must be 64, 128 or 256";
-        case INTFA_ERR_SEQLEN: return "seqlen must be positive";
+        case INTFA_ERR_SEQLEN: return "seqlen must be positive; seqlen_k, when set, must equal it for causal attention";
         case INTFA_ERR_ALIGN: return "pointers and row/head/batch strides must be 16-byte aligned";
         case INTFA_ERR_DTYPE: return "unknown dtype enum";
         case INTFA_ERR_WORKSPACE: return "workspace missing, misaligned or too small for num_splits";

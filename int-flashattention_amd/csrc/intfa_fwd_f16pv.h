@@ -91,7 +91,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     const int hk = h / kv_group;                     // K/V head of this query head
     // ragged sequence lengths are handled as in the full-int8 kernel (zero-filled copies, masked last block, rows past
     // the end computed on clamped inputs and not stored)
-    const int nb_total = (p.seqlen + BN - 1) / BN;
+    const int nb_total = (p.seqlen_k + BN - 1) / BN;
     int nb_begin = 0, nb_end = CAUSAL ? ((mb + 1) * RDIAG < nb_total ? (mb + 1) * RDIAG : nb_total) : nb_total;
     if (SPLIT) {
         nb_begin = split * p.blocks_per_split;
@@ -122,8 +122,8 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     // ---- global -> LDS copies
     const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
     const char* Vg = p.v + b * p.v_sb + hk * p.v_sh;
-    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen - 1) * p.k_sn + KROW));
-    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + VROW));
+    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen_k - 1) * p.k_sn + KROW));
+    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen_k - 1) * p.v_sn + VROW));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
     const auto k_lane = tile_load_lane<KROW, SWZ_K, BN>(k_sn, wave, lane);
     const auto v_lane = tile_load_lane<VROW, SWZ_V16, BN>(v_sn, wave, lane);
@@ -138,7 +138,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
         if (!QK_INT8 || tid >= BN) return 0u;
         int key = nb * BN + tid;
-        key = key < p.seqlen ? key : p.seqlen - 1;                                    // keys past the end are masked later
+        key = key < p.seqlen_k ? key : p.seqlen_k - 1;                                    // keys past the end are masked later
         const char* src = Ksg + (int64_t)key * ks_stride;
         if (p.scale_dtype == 2) return *(const uint32_t*)src;
         return (uint32_t)*(const uint16_t*)src;
@@ -321,7 +321,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
             if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
         }
         const int diag_begin = mb * RDIAG;
-        const int tail_keys = p.seqlen - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
+        const int tail_keys = p.seqlen_k - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
         const bool ragged = !CAUSAL && tail_keys < BN && nb_end == nb_total;
         const int plain_end = CAUSAL ? (nb_end > diag_begin ? diag_begin : nb_end) : (ragged ? nb_end - 1 : nb_end);
         int nb = nb_begin;

@@ -102,7 +102,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     // Sequence lengths that are not a multiple of the block sizes: the copies of K/V rows past the end return zeros
     // (bounds-checked buffer loads), the last key block runs the masked code instance, query rows past the end are
     // computed on clamped inputs and not stored.
-    const int nb_total = (p.seqlen + BN - 1) / BN;
+    const int nb_total = (p.seqlen_k + BN - 1) / BN;
     int nb_begin = 0, nb_end = CAUSAL ? ((mb + 1) * RDIAG < nb_total ? (mb + 1) * RDIAG : nb_total) : nb_total;
     if (SPLIT) {
         nb_begin = split * p.blocks_per_split;
@@ -133,8 +133,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     // ---- global -> LDS copies (asynchronous, straight into LDS)
     const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
     const char* Vg = DUMP_S ? Kg : p.v + b * p.v_sb + hk * p.v_sh + half * DV;
-    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen - 1) * p.k_sn + D));
-    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen - 1) * p.v_sn + DV));
+    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen_k - 1) * p.k_sn + D));
+    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen_k - 1) * p.v_sn + DV));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
     const auto k_lane = tile_load_lane<D, SWZ_K, BN>(k_sn, wave, lane);
     const auto v_lane = tile_load_lane<DV, SWZ_V8, BN>(v_sn, wave, lane);
@@ -169,7 +169,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {           // raw bits
         if (DUMP_S) return 0u;
         int key = nb * BN + ks_key;
-        key = key < p.seqlen ? key : p.seqlen - 1;                                    // keys past the end are masked later
+        key = key < p.seqlen_k ? key : p.seqlen_k - 1;                                    // keys past the end are masked later
         const char* src = Ksg + (int64_t)key * ks_stride;
         if (p.scale_dtype == 2) return *(const uint32_t*)src;
         return (uint32_t)*(const uint16_t*)src;
@@ -275,11 +275,11 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             v16i& nacc = sacc[(st + 1) & 1];
             if (DUMP_S) {
                 const int key0 = nb * BN + 32 * st;
-                int32_t* srow = p.s_dump + ((int64_t)(b * p.heads + h) * p.seqlen + q_ld) * p.seqlen + key0;
+                int32_t* srow = p.s_dump + ((int64_t)(b * p.heads + h) * p.seqlen + q_ld) * p.seqlen_k + key0;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int kidx = 8 * (r >> 2) + 4 * lh + (r & 3);
-                    if (q_valid && key0 + kidx < p.seqlen) srow[kidx] = acc[r];
+                    if (q_valid && key0 + kidx < p.seqlen_k) srow[kidx] = acc[r];
                 }
             }
 #pragma unroll
@@ -422,7 +422,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
         }
         const int diag_begin = mb * RDIAG;                 // first key block that touches the diagonal
-        const int tail_keys = p.seqlen - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
+        const int tail_keys = p.seqlen_k - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
         const bool ragged = !CAUSAL && tail_keys < BN && nb_end == nb_total;
         const int plain_end = CAUSAL ? (nb_end > diag_begin ? diag_begin : nb_end) : (ragged ? nb_end - 1 : nb_end);
         int nb = nb_begin;

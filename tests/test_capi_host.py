@@ -68,6 +68,7 @@ def _valid_block():
     (lambda p: setattr(p, "v_scale", None), -1),
     (lambda p: setattr(p, "head_dim", 48), -2),
     (lambda p: setattr(p, "seqlen", -128), -3),
+    (lambda p: (setattr(p, "causal", 1), setattr(p, "seqlen_k", 512)), -3),    # causal with a different key length
     (lambda p: setattr(p, "seqlen", 0), -3),
     (lambda p: setattr(p, "k", 0x10008), -4),
     (lambda p: setattr(p, "q_stride_n", 120), -4),

@@ -348,6 +348,45 @@ def test_ragged_outputs_do_not_touch_memory_past_the_end():
     assert torch.equal(big[:, :, :130], o) and (big[:, :, 130:] == 7.0).all()
 
 
+# ------------------------------------------------------------------------------------------ separate key length
+def _dense_cross(q, k, v, sm):
+    s = torch.matmul(q.float(), k.float().transpose(2, 3)) * sm
+    return torch.matmul(torch.softmax(s, dim=-1), v.float())
+
+
+@pytest.mark.parametrize("B,H,Nq,Nk,D", [(2, 4, 1, 1000, 128), (1, 2, 128, 384, 64), (1, 3, 200, 77, 128), (1, 2, 130, 2048, 256)])
+def test_separate_query_and_key_lengths(B, H, Nq, Nk, D):
+    """Non-causal attention with Nq != Nk (decoding against a cache, cross attention): there is no oracle restatement
+    with two lengths, so the check is the mathematics itself - int32 S against an integer matmul, outputs against dense
+    softmax attention on the dequantised inputs within the quantisation error the equal-length cases show."""
+    g = torch.Generator().manual_seed(70)
+    q = torch.randn((B, H, Nq, D), generator=g).half()
+    k = torch.randn((B, H, Nk, D), generator=g).half()
+    v = torch.randn((B, H, Nk, D), generator=g).half()
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    sm = D ** -0.5
+    s = M.debug_qk_int32(*gpu(q8, k8)).cpu()
+    assert s.shape == (B, H, Nq, Nk) and torch.equal(s, O.qk_int32(q8, k8))
+    exact = _dense_cross(q, k, v, sm)
+    o = M.attention(*gpu(q, k, v), False, sm)
+    assert o.shape == (B, H, Nq, D) and max_abs(o, exact) <= 2e-3
+    qd, kd = q8.float() * qs.float()[..., None], k8.float() * ks.float()[..., None]
+    o = M.attention_int8(*gpu(q8, k8, v, qs, ks), False, sm)
+    assert max_abs(o, _dense_cross(qd, kd, v, sm)) <= 3e-3          # same dequantised Q, K: only fp16 P and output rounding
+    vd = v8.float() * vs.float()[..., None, None]
+    o = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm)
+    assert max_abs(o, _dense_cross(qd, kd, vd, sm)) <= 3e-2 and mean_rel(o, _dense_cross(qd, kd, vd, sm)) <= 4e-2   # + P8 quantisation
+    o2 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm, num_splits=3)
+    assert max_abs(o2, o) <= 2e-2
+
+
+def test_causal_needs_equal_lengths():
+    q = torch.zeros((1, 1, 128, 64), dtype=torch.float16, device=DEV)
+    k = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device=DEV)
+    with pytest.raises(ValueError, match="causal"):
+        M.attention(q, k, k, True, 1.0)
+
+
 # ------------------------------------------------------------------------------------------ grouped K/V heads
 @pytest.mark.parametrize("variant", ["full", "half", "fp"])
 @pytest.mark.parametrize("B,H,H_kv,N,D,causal", [(1, 8, 2, 256, 128, True), (2, 16, 16 // 4, 384, 64, False), (2, 4, 1, 256, 128, True)])
