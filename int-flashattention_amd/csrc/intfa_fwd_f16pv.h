@@ -354,7 +354,9 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     if (SPLIT) {
         const int64_t row = ((int64_t)(split * pe->batch + eb) * e_heads + eh) * e_seqlen + q_row;
         float* op = pe->o_part + row * D;
-        const bool seen = nb_begin < nb_end;
+        // a row contributes nothing to this split when the split's range is empty for its workgroup, or when every
+        // block of the range lies above the row's diagonal (its wave skipped them: the running max is still -inf)
+        const bool seen = nb_begin < nb_end && m_run > -INFINITY;
         if (q_valid) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)

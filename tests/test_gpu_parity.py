@@ -256,6 +256,26 @@ def test_half_and_fp_split_kv_equals_single_pass(variant, causal, splits, D):
     assert (l1 - l2).abs().max().item() <= 1e-3
 
 
+@pytest.mark.parametrize("variant,N,D,splits", [("fp", 128, 64, 5), ("half", 384, 128, 2), ("full", 256, 256, 4), ("fp", 511, 256, 3)])
+def test_causal_split_that_starts_inside_the_diagonal(variant, N, D, splits):
+    """A split whose key range begins inside a query block's diagonal region holds no key at all for that block's first
+    rows (their waves skip every block of the range): those rows must contribute nothing, not NaN."""
+    x = quantised(2, 2, N, D, seed=37)
+    sm = D ** -0.5
+    if variant == "fp":
+        o = M.attention(*gpu(x["q"], x["k"], x["v"]), True, sm, num_splits=splits)
+        ref = O.attention_fp(x["q"], x["k"], x["v"], True, sm, block_n=64)
+    elif variant == "half":
+        o = M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), True, sm, num_splits=splits)
+        ref = O.attention_int8(x["q8"], x["k8"], x["v"], x["qs"], x["ks"], True, sm, block_n=64)
+    else:
+        o = run_full(x, True, sm, num_splits=splits, p_round="reference")
+        ref = O.attention_full_int8_splitkv(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], True, sm, splits,
+                                            block_n=M.block_n("full", D))
+    assert torch.isfinite(o).all()
+    assert max_abs(o, ref) <= 4e-3 and mean_rel(o, ref) <= 3e-4
+
+
 def test_half_int8_lse_matches_oracle():
     x = quantised(1, 2, 256, 128, seed=35)
     _, lse = M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), True, 0.09, return_lse=True)
