@@ -30,6 +30,8 @@ WORKLOADS = {
     "fp16_B4_H32_N4096_d128": dict(variant="fp", B=4, H=32, N=4096, D=128, causal=False, splits=1),
     "full_int8_B1_H32_N16384_d128_causal_splitkv": dict(variant="full", B=1, H=32, N=16384, D=128, causal=True, splits=2,
                                                         k_outlier_frac=0.01),
+    "full_int8_B1_H32_N16384_d128_causal": dict(variant="full", B=1, H=32, N=16384, D=128, causal=True, splits=1,
+                                                k_outlier_frac=0.01),
     "full_int8_B16_H16_N1024_d64_bf16": dict(variant="full", B=16, H=16, N=1024, D=64, causal=False, splits=1,
                                              dtype="bfloat16", std=0.5),
     "full_int8_B16_H16_N1024_d256_bf16": dict(variant="full", B=16, H=16, N=1024, D=256, causal=False, splits=1,

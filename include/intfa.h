@@ -118,6 +118,13 @@ const char* intfa_error_string(int code);
  * so a bit-faithful CPU evaluation must use the same value.  Negative INTFA_ERR_* for unknown arguments. */
 int intfa_fwd_block_n(int variant, int head_dim);
 
+/* A split count for the problem in *p (its num_splits and workspace members are ignored): 1 when the single-pass grid
+ * already fills the GPU, otherwise enough splits to reach about two workgroups per compute unit while leaving every split
+ * at least four key blocks; the counterpart of the heuristic that lives in the reference's absent flash_api.cpp
+ * (csrc/flash_fwd_launch_template.h:193-253 only consumes it).  variant: INTFA_VARIANT_*; num_cus: compute units of
+ * the device, 0 = 256 (MI355X).  Negative INTFA_ERR_* for a rejected block. */
+int intfa_fwd_suggest_splits(const intfa_fwd_params* p, int variant, int num_cus);
+
 /* Bytes of workspace the forward needs for p->num_splits (0 when num_splits <= 1). */
 size_t intfa_fwd_workspace_bytes(const intfa_fwd_params* p);
 

@@ -37,7 +37,7 @@ class FwdParams(ctypes.Structure):
 
 VARIANT_FULL_INT8, VARIANT_HALF_INT8, VARIANT_FP16 = 0, 1, 2
 
-EXPORTS = ("intfa_version", "intfa_error_string", "intfa_fwd_block_n", "intfa_fwd_workspace_bytes",
+EXPORTS = ("intfa_version", "intfa_error_string", "intfa_fwd_block_n", "intfa_fwd_workspace_bytes", "intfa_fwd_suggest_splits",
            "intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16", "intfa_debug_qk_int32",
            "intfa_quant_pertoken", "intfa_quant_pertensor_workspace_bytes", "intfa_quant_pertensor")
 
@@ -61,6 +61,8 @@ def load():
     lib.intfa_fwd_block_n.argtypes = [ctypes.c_int, ctypes.c_int]
     lib.intfa_error_string.restype = ctypes.c_char_p
     lib.intfa_error_string.argtypes = [ctypes.c_int]
+    lib.intfa_fwd_suggest_splits.restype = ctypes.c_int
+    lib.intfa_fwd_suggest_splits.argtypes = [pp, ctypes.c_int, ctypes.c_int]
     lib.intfa_fwd_workspace_bytes.restype = ctypes.c_size_t
     lib.intfa_fwd_workspace_bytes.argtypes = [pp]
     for name in ("intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16"):

@@ -98,6 +98,11 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
     p.causal = 1 if causal else 0
     p.sm_scale = float(sm_scale)
     p.p_round = p_round
+    if num_splits == "auto":
+        cus = torch.cuda.get_device_properties(q.device).multi_processor_count
+        num_splits = lib.intfa_fwd_suggest_splits(ctypes.byref(p), _VARIANT_ENUM[variant], cus)
+        if num_splits < 0:
+            _capi.check(num_splits, "intfa_fwd_suggest_splits")
     p.num_splits = int(num_splits)
     ws = None
     if p.num_splits > 1:

@@ -175,6 +175,26 @@ const char* intfa_error_string(int code) {
 
 size_t intfa_fwd_workspace_bytes(const intfa_fwd_params* p) { return workspace_bytes_for(p); }
 
+int intfa_fwd_suggest_splits(const intfa_fwd_params* p, int variant, int num_cus) {
+    if (p == nullptr) return INTFA_ERR_NULL;
+    if (variant < INTFA_VARIANT_FULL_INT8 || variant > INTFA_VARIANT_FP16) return INTFA_ERR_DTYPE;
+    if (p->batch <= 0 || p->heads <= 0) return INTFA_ERR_SHAPE;
+    if (p->seqlen <= 0 || p->seqlen_k < 0) return INTFA_ERR_SEQLEN;
+    if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256) return INTFA_ERR_HEAD_DIM;
+    const int cus = num_cus > 0 ? num_cus : 256;
+    const int64_t slots = 2ll * cus;                                           // two workgroups per compute unit
+    int64_t wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kBlockM - 1) / kBlockM);
+    if (variant == INTFA_VARIANT_FULL_INT8 && p->head_dim == 256) wgs *= 2;     // column halves
+    if (wgs * 5 >= slots * 4) return 1;                                        // at least 80 % of the slots are used anyway
+    const int seqlen_k = p->seqlen_k > 0 ? p->seqlen_k : p->seqlen;
+    const int bn = block_n_for(variant, p->head_dim);
+    const int64_t blocks = (seqlen_k + bn - 1) / bn;
+    int64_t splits = (slots + wgs - 1) / wgs;
+    if (splits > blocks / 4) splits = blocks / 4;                              // keep four key blocks per split
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    return splits < 1 ? 1 : (int)splits;
+}
+
 int intfa_fwd_full_int8(const intfa_fwd_params* p, void* stream) {
     return run_forward(INTFA_VARIANT_FULL_INT8, p, 1, 1, true, true, (hipStream_t)stream);
 }

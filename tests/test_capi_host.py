@@ -119,6 +119,24 @@ def test_entry_points_keep_the_reference_asserts():
         M.attention_full_int8(q, q, q, s, s, torch.ones((1, 1), dtype=torch.float16), False, 1.0)
 
 
+def test_split_count_heuristic():
+    lib = _capi.load()
+    p = _capi.FwdParams()
+    p.batch, p.heads, p.seqlen, p.head_dim = 4, 32, 4096, 128
+    assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 0, 256) == 1              # 4096 workgroups fill 256 CUs
+    p.batch, p.heads, p.seqlen, p.seqlen_k = 1, 8, 1, 8192                          # decoding: 8 workgroups
+    assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 0, 256) == 16             # 64 key blocks, four per split
+    assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 1, 256) == 32             # 64-key blocks: 128 of them
+    assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 0, 0) == 16               # default device size
+    p.seqlen_k = 256
+    assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 0, 256) == 1              # too few key blocks to split
+    p.batch, p.heads, p.seqlen, p.seqlen_k = 1, 32, 1024, 0
+    assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 0, 256) == 2              # 256 workgroups on 512 slots
+    assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 7, 256) == -5 and lib.intfa_fwd_suggest_splits(None, 0, 256) == -1
+    p.head_dim = 100
+    assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 0, 256) == -2
+
+
 def test_quantisers_refuse_cpu_tensors_and_bad_arguments():
     x = torch.randn((2, 3, 16, 32)).half()
     for fn in (M.quant_pertoken, M.quant_pertensor):

@@ -400,6 +400,24 @@ def test_separate_query_and_key_lengths(B, H, Nq, Nk, D):
     assert max_abs(o2, o) <= 2e-2
 
 
+def test_decoding_shape_with_automatic_splits():
+    """One query against a long cache: num_splits="auto" spreads the keys over many workgroups; the result equals the
+    single pass (no P requantisation on the half-int8 path) and stays within the P8 noise on the full-int8 path."""
+    g = torch.Generator().manual_seed(71)
+    B, H, Nk, D = 1, 8, 8192, 128
+    q = torch.randn((B, H, 1, D), generator=g).half()
+    k = torch.randn((B, H, Nk, D), generator=g).half()
+    v = torch.randn((B, H, Nk, D), generator=g).half()
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    sm = D ** -0.5
+    a1 = M.attention_int8(*gpu(q8, k8, v, qs, ks), False, sm)
+    a2 = M.attention_int8(*gpu(q8, k8, v, qs, ks), False, sm, num_splits="auto")
+    assert max_abs(a2, a1) <= 1e-3
+    f1 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm)
+    f2 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm, num_splits="auto")
+    assert max_abs(f2, f1) <= 2e-2 and max_abs(f2, _dense_cross(q, k, v, sm)) <= 3e-2
+
+
 def test_causal_needs_equal_lengths():
     q = torch.zeros((1, 1, 128, 64), dtype=torch.float16, device=DEV)
     k = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device=DEV)
