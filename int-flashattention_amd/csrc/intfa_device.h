@@ -2,7 +2,7 @@
 //
 // Tile geometry used throughout:
 //   * a workgroup is 4 wavefronts (256 threads) and owns BLOCK_M = 128 query rows, 32 per wavefront;
-//   * keys are consumed in blocks of BLOCK_N = 128, each handled as 4 sub-tiles of 32 keys;
+//   * keys are consumed in blocks of 128 or 64 (per kernel and head_dim), each handled as sub-tiles of 32 keys;
 //   * the score tile is computed TRANSPOSED, S^T = K Q^T, with v_mfma_i32_32x32x32_i8: a lane then holds one
 //     query column (lane % 32) and 16 keys, so row max / row sum are in-lane reductions plus one exchange
 //     between lane l and lane l^32, and the accumulator registers run along the key axis - the contraction
@@ -35,7 +35,6 @@ typedef short v4s __attribute__((ext_vector_type(4)));
 #define INTFA_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
 
 constexpr int kBlockM = 128;
-constexpr int kBlockN = 128;                  // key block of the full-int8 kernel for head_dim <= 128
 constexpr int kThreads = 256;
 constexpr float kLog2_127 = 6.98868468677f;   // log2(127)
 

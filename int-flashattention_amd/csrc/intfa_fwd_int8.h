@@ -1,7 +1,7 @@
 // Forward kernel with int8 Q K^T and int8 P V (full-int8).
 //
-// Algorithm restated from the reference tile loop (flash_atten_full_int8.py:9-71): per key block of kBlockN
-// keys, S = Q8 K8^T in int32; X = S * q_scale[row] * k_scale[col]; running max m in the exp2 domain;
+// Algorithm restated from the reference tile loop (flash_atten_full_int8.py:9-71): per key block of BN keys
+// (FullInt8Geom below), S = Q8 K8^T in int32; X = S * q_scale[row] * k_scale[col]; running max m in the exp2 domain;
 // P = exp2(X * c - m_new); l sums the UNQUANTISED P; P is requantised to int8 with the fixed scale 127;
 // acc = acc * alpha + P8 V8; output acc * v_scale / (127 l).
 // Differences in evaluation order that stay within fp32 rounding: q_scale * c is folded into one per-row
