@@ -43,6 +43,11 @@ def _pad_head_dim(t: torch.Tensor, d_to: int) -> torch.Tensor:
     return t if d == d_to else F.pad(t, (0, d_to - d))
 
 
+def _can_fold(t: torch.Tensor, n: int) -> bool:
+    """True if the rows of consecutive heads of t ([Z, H, N, ...]) lie at one constant stride."""
+    return n == 1 or t.stride(1) == n * t.stride(2)
+
+
 def _require_gpu(*ts):
     for t in ts:
         if t is not None and not t.is_cuda:
@@ -94,6 +99,15 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
     p.batch, p.heads, p.seqlen, p.head_dim = Z, H, N, dk
     p.heads_kv = H_kv
     p.seqlen_k = N_k
+    # Few queries per head with grouped K/V heads (decoding): the g query heads of a group become g*N rows of ONE head,
+    # so that a group streams its K/V once instead of g times.  Pure re-striding: same memory, same results per row.
+    g = H // H_kv
+    if g > 1 and not causal and g * N <= 2 * BLOCK and _can_fold(q_, N) and (variant == "fp" or _can_fold(q_scale, N)):
+        p.heads, p.heads_kv, p.seqlen = H_kv, H_kv, g * N
+        p.q_stride_h, p.q_stride_n = g * q_.stride(1), (q_.stride(2) if N > 1 else q_.stride(1))
+        p.o_stride_h = g * out.stride(1)
+        if variant != "fp":
+            p.qs_stride_h, p.qs_stride_n = g * q_scale.stride(1), (q_scale.stride(2) if N > 1 else q_scale.stride(1))
     p.io_dtype = _TORCH_TO_ENUM[out_dtype]
     p.causal = 1 if causal else 0
     p.sm_scale = float(sm_scale)

@@ -418,6 +418,31 @@ def test_decoding_shape_with_automatic_splits():
     assert max_abs(f2, f1) <= 2e-2 and max_abs(f2, _dense_cross(q, k, v, sm)) <= 3e-2
 
 
+@pytest.mark.parametrize("Nq", [1, 3, 16])
+def test_grouped_decoding_folds_heads_into_rows(Nq):
+    """Grouped K/V heads with few queries: the wrapper runs a group's heads as rows of one head; every row's result must
+    equal ordinary attention on repeated K/V, LSE included."""
+    g_ = torch.Generator().manual_seed(72)
+    B, H, Hkv, Nk, D = 2, 16, 4, 1500, 128
+    q = torch.randn((B, H, Nq, D), generator=g_).half()
+    k = torch.randn((B, Hkv, Nk, D), generator=g_).half()
+    v = torch.randn((B, Hkv, Nk, D), generator=g_).half()
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    rep = lambda t: t.repeat_interleave(H // Hkv, dim=1)
+    sm = D ** -0.5
+    o, lse = M.attention(*gpu(q, k, v), False, sm, return_lse=True)
+    exact = _dense_cross(q, rep(k), rep(v), sm)
+    assert o.shape == (B, H, Nq, D) and max_abs(o, exact) <= 2e-3
+    s = torch.matmul(q.float(), rep(k).float().transpose(2, 3)) * sm * 1.44269504
+    assert (lse.cpu() - torch.logsumexp(s * 0.6931471805599453, dim=-1) * 1.44269504).abs().max().item() < 2e-3
+    qd, kd = q8.float() * qs.float()[..., None], k8.float() * ks.float()[..., None]
+    o = M.attention_int8(*gpu(q8, k8, v, qs, ks), False, sm, num_splits="auto")
+    assert max_abs(o, _dense_cross(qd, rep(kd), rep(v), sm)) <= 3e-3
+    o = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm)
+    o_rep = M.attention_full_int8(*gpu(q8, rep(k8), rep(v8), qs, rep(ks), rep(vs)), False, sm)     # ungrouped call
+    assert torch.equal(o, o_rep)
+
+
 def test_causal_needs_equal_lengths():
     q = torch.zeros((1, 1, 128, 64), dtype=torch.float16, device=DEV)
     k = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device=DEV)
