@@ -92,7 +92,8 @@ int setup_split(const intfa_fwd_params* p, int block_n, KParams* kp) {
 
 int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t stream) {
     const int64_t rows = (int64_t)kp.batch * kp.heads * kp.seqlen;
-    const int grid = (int)((rows + 3) / 4);       // one wave per output row, 4 rows per workgroup
+    const int rpb = 256 / (kp.head_dim / 4);      // head_dim / 4 lanes per output row
+    const int grid = (int)((rows + rpb - 1) / rpb);
 #define INTFA_COMBINE(DD, ODT) hipLaunchKernelGGL((splitkv_combine_kernel<DD, ODT>), dim3(grid), dim3(256), 0, stream, kp)
     if (kp.head_dim == 64) { if (p->io_dtype == INTFA_F16) INTFA_COMBINE(64, 0); else INTFA_COMBINE(64, 1); }
     else if (kp.head_dim == 128) { if (p->io_dtype == INTFA_F16) INTFA_COMBINE(128, 0); else INTFA_COMBINE(128, 1); }

@@ -5,43 +5,55 @@
 
 namespace intfa {
 
-// One wavefront per output row: lane l owns head_dim/64 ... elements; 4 rows per 256-thread workgroup.
+// D / 4 lanes per output row (one 16-byte load per lane and split, one 8-byte store), 256 / (D / 4) rows per workgroup;
+// the loads of four splits are in flight together.
 template <int D, int OUT_DT>
 __global__ void __launch_bounds__(256) splitkv_combine_kernel(const KParams p) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int LPR = D / 4, RPB = 256 / LPR;
+    const int sub = threadIdx.x % LPR, rl = threadIdx.x / LPR;
     const int64_t rows = (int64_t)p.batch * p.heads * p.seqlen;
-    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    const int64_t row = (int64_t)blockIdx.x * RPB + rl;
     if (row >= rows) return;
     const int ns = p.num_splits;
-    // log-sum-exp over splits (every lane computes the same scalars)
+    // log-sum-exp over splits (every lane of a row computes the same scalars)
     float lse_max = -INFINITY;
     for (int s = 0; s < ns; ++s) lse_max = fmaxf(lse_max, p.lse_part[(int64_t)s * rows + row]);
     if (lse_max == -INFINITY) lse_max = 0.f;
     float sum = 0.f;
     for (int s = 0; s < ns; ++s) sum += fast_exp2(p.lse_part[(int64_t)s * rows + row] - lse_max);
     const float lse = (sum == 0.f || sum != sum) ? INFINITY : __builtin_log2f(sum) + lse_max;
-    constexpr int PER = D / 64;                     // consecutive elements per lane
-    float acc[PER];
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    const float* op0 = p.o_part + row * D + sub * 4;
+    const int64_t sstride = rows * D;
+    for (int s0 = 0; s0 < ns; s0 += 4) {
+        v4f part[4];
+        float w[4];
 #pragma unroll
-    for (int i = 0; i < PER; ++i) acc[i] = 0.f;
-    for (int s = 0; s < ns; ++s) {
-        const float w = fast_exp2(p.lse_part[(int64_t)s * rows + row] - lse);
-        const float* op = p.o_part + ((int64_t)s * rows + row) * D + lane * PER;
+        for (int u = 0; u < 4; ++u) {
+            const int s = s0 + u < ns ? s0 + u : ns - 1;                 // clamped loads, zero weight past the end
+            part[u] = *(const v4f*)(op0 + (int64_t)s * sstride);
+            w[u] = s0 + u < ns ? fast_exp2(p.lse_part[(int64_t)s * rows + row] - lse) : 0.f;
+        }
 #pragma unroll
-        for (int i = 0; i < PER; ++i) acc[i] = fmaf(w, op[i], acc[i]);
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = fmaf(w[u], part[u][i], acc[i]);
     }
     const int64_t bh = row / p.seqlen, n = row % p.seqlen;
     const int64_t b = bh / p.heads, h = bh % p.heads;
-    char* orow = p.out + b * p.o_sb + h * p.o_sh + n * p.o_sn + lane * PER * 2;
+    char* orow = p.out + b * p.o_sb + h * p.o_sh + n * p.o_sn + sub * 8;
+    if (OUT_DT == 0) {
+        v4h o;
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-        if (OUT_DT == 0) {
-            ((_Float16*)orow)[i] = (_Float16)acc[i];
-        } else {
-            ((uint16_t*)orow)[i] = (uint16_t)f32_to_bf16_bits(acc[i]);
-        }
+        for (int i = 0; i < 4; ++i) o[i] = (_Float16)acc[i];
+        *(v4h*)orow = o;
+    } else {
+        v4s o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = (short)f32_to_bf16_bits(acc[i]);
+        *(v4s*)orow = o;
     }
-    if (p.lse != nullptr && lane == 0) p.lse[row] = lse;
+    if (p.lse != nullptr && sub == 0) p.lse[row] = lse;
 }
 
 }  // namespace intfa
