@@ -94,7 +94,9 @@ typedef struct intfa_fwd_params {
     float   sm_scale;
     int32_t p_round;          /* INTFA_PROUND_* (full-int8 only) */
 
-    int32_t num_splits;       /* <= 1: single pass; > 1: split-KV partials + combine (needs workspace) */
+    int32_t num_splits;       /* <= 1: single pass; > 1: split-KV partials + combine (needs workspace).  The key blocks
+                                 are dealt evenly to the splits; with causal, per query block of 128 rows, the blocks
+                                 visible to it */
     void*   workspace;        /* device scratch of at least intfa_fwd_workspace_bytes() bytes, or NULL */
     size_t  workspace_bytes;
 

@@ -94,8 +94,11 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     const int nb_total = (p.seqlen_k + BN - 1) / BN;
     int nb_begin = 0, nb_end = CAUSAL ? ((mb + 1) * RDIAG < nb_total ? (mb + 1) * RDIAG : nb_total) : nb_total;
     if (SPLIT) {
-        nb_begin = split * p.blocks_per_split;
-        const int e = nb_begin + p.blocks_per_split;
+        // non-causal: the key blocks of the sequence are dealt evenly to the splits (csrc/flash_fwd_kernel.h:503-511);
+        // causal: the blocks VISIBLE to this query block are, so that no split of a query block is empty or short
+        const int per = CAUSAL ? (nb_end + n_split - 1) / n_split : p.blocks_per_split;
+        nb_begin = split * per;
+        const int e = nb_begin + per;
         nb_end = e < nb_end ? e : nb_end;
     }
     const int q_row = mb * kBlockM + wave * 32 + lq;

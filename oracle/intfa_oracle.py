@@ -137,15 +137,18 @@ def p_requant_rne(p: torch.Tensor) -> torch.Tensor:
 # --------------------------------------------------------------------------------------------------
 def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float,
                      block_m: int, block_n: int, key_lo: int = 0, key_hi: Optional[int] = None,
-                     p_requant=p_requant_reference, pv_dtype=torch.float16):
+                     p_requant=p_requant_reference, pv_dtype=torch.float16,
+                     row_lo: int = 0, row_hi: Optional[int] = None):
     """Runs the reference's tile loop over key blocks [key_lo, key_hi) for every query row at once.
 
     Rows are grouped in tiles of ``block_m`` as the reference's programs are; for a causal run a tile sees
     the key blocks below its first row without a mask (stage 1) and the blocks of its own row range with the
     mask (stage 2), flash_atten_full_int8.py:18-25.  Returns fp32 (acc, l, m) with acc un-normalised.
+    Only rows [row_lo, row_hi) are evaluated (the others keep m = -inf, l = 1, acc = 0).
     """
     B, H, N, D = q.shape
     key_hi = N if key_hi is None else key_hi
+    row_hi = N if row_hi is None else row_hi
     # N need not be a multiple of the blocks: the last key block and the last row tile are simply shorter, which is
     # what masking the missing keys with -inf amounts to (csrc/mask.h:261-263 for the reference's CUDA tree; its Triton
     # kernels have no bounds handling at all)
@@ -172,6 +175,7 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
         else:
             segments = [(0, N, False)]
         for r0, r1, masked in segments:
+            r0, r1 = max(r0, row_lo), min(r1, row_hi)
             if r0 >= r1:
                 continue
             qi = q[:, :, r0:r1]
@@ -266,22 +270,41 @@ def splitkv_combine(o_parts: torch.Tensor, lse_parts: torch.Tensor) -> Tuple[tor
     return (w[..., None] * o_parts).sum(dim=0), lse
 
 
+def splitkv_ranges_causal(n_keys: int, block_m: int, block_n: int, num_splits: int):
+    """Causal split-KV as the kernels do it: per row tile of block_m rows, the key blocks VISIBLE to the tile are dealt
+    evenly to the splits.  Returns [(row_lo, row_hi, [(block_min, block_max) per split])] per tile."""
+    n_blocks = (n_keys + block_n - 1) // block_n
+    out = []
+    for r0 in range(0, n_keys, block_m):
+        vis = min((r0 + block_m + block_n - 1) // block_n, n_blocks)
+        per = (vis + num_splits - 1) // num_splits
+        out.append((r0, min(r0 + block_m, n_keys), [(s * per, min(vis, (s + 1) * per)) for s in range(num_splits)]))
+    return out
+
+
 def attention_full_int8_splitkv(q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float, num_splits: int, *,
                                 block_m: int = 128, block_n: int = 128, out_dtype=torch.float16):
-    """Full-int8 forward evaluated as ``num_splits`` independent key ranges merged by ``splitkv_combine``."""
+    """Full-int8 forward evaluated as ``num_splits`` independent key ranges merged by ``splitkv_combine``: the ranges of
+    ``splitkv_ranges`` for a non-causal pass, those of ``splitkv_ranges_causal`` (per row tile) for a causal one."""
     B, H, N, D = q.shape
-    o_parts, lse_parts = [], []
-    for b0, b1 in splitkv_ranges(N, block_n, num_splits):
+    o_parts = torch.zeros((num_splits, B, H, N, D))
+    lse_parts = torch.full((num_splits, B, H, N), float("-inf"))
+    if causal:
+        jobs = [(s, r0, r1, b0, b1) for r0, r1, ranges in splitkv_ranges_causal(N, block_m, block_n, num_splits)
+                for s, (b0, b1) in enumerate(ranges)]
+    else:
+        jobs = [(s, 0, N, b0, b1) for s, (b0, b1) in enumerate(splitkv_ranges(N, block_n, num_splits))]
+    for s, r0, r1, b0, b1 in jobs:
         if b0 >= b1:
-            o_parts.append(torch.zeros((B, H, N, D)))
-            lse_parts.append(torch.full((B, H, N), float("-inf")))
             continue
         acc, l, m = _blocked_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale,
-                                     block_m, block_n, key_lo=b0 * block_n, key_hi=min(b1 * block_n, N))
-        seen = ~torch.isinf(m)                       # causal rows above the split's range saw no key
-        o_parts.append(torch.where(seen[..., None], acc / l[..., None], torch.zeros_like(acc)))
-        lse_parts.append(torch.where(seen, m + torch.log2(l), torch.full_like(m, float("-inf"))))
-    o, _ = splitkv_combine(torch.stack(o_parts), torch.stack(lse_parts))
+                                     block_m, block_n, key_lo=b0 * block_n, key_hi=min(b1 * block_n, N),
+                                     row_lo=r0, row_hi=r1)
+        seen = ~torch.isinf(m[:, :, r0:r1])          # rows above the split's range saw no key
+        a, ll, mm = acc[:, :, r0:r1], l[:, :, r0:r1], m[:, :, r0:r1]
+        o_parts[s, :, :, r0:r1] = torch.where(seen[..., None], a / ll[..., None], torch.zeros_like(a))
+        lse_parts[s, :, :, r0:r1] = torch.where(seen, mm + torch.log2(ll), torch.full_like(mm, float("-inf")))
+    o, _ = splitkv_combine(o_parts, lse_parts)
     return o.to(out_dtype)
 
 

@@ -291,6 +291,18 @@ def test_splitkv_combine_reproduces_dense_softmax():
     assert (lse - torch.logsumexp(x, dim=-1) * O.LOG2E).abs().max() < 1e-4
 
 
+def test_causal_split_ranges_cover_each_tiles_visible_blocks_once():
+    for n, bm, bn, ns in ((1024, 128, 128, 3), (1000, 128, 64, 4), (256, 128, 64, 5), (130, 128, 128, 2)):
+        n_blocks = -(-n // bn)
+        for r0, r1, ranges in O.splitkv_ranges_causal(n, bm, bn, ns):
+            vis = min(-(-(r0 + bm) // bn), n_blocks)                 # blocks that hold a key <= the tile's last row
+            covered = [b for b0, b1 in ranges for b in range(b0, b1)]
+            assert covered == list(range(vis)) and len(ranges) == ns
+            assert max(b1 - b0 for b0, b1 in ranges) == -(-vis // ns)
+    assert O.splitkv_ranges_causal(512, 128, 128, 2) == [(0, 128, [(0, 1), (1, 1)]), (128, 256, [(0, 1), (1, 2)]),
+                                                         (256, 384, [(0, 2), (2, 3)]), (384, 512, [(0, 2), (2, 4)])]
+
+
 def test_splitkv_ranges_follow_ceil_partition():
     assert O.splitkv_ranges(1024, 128, 3) == [(0, 3), (3, 6), (6, 8)]
     assert O.splitkv_ranges(256, 128, 4) == [(0, 1), (1, 2), (2, 2), (3, 2)]
