@@ -192,8 +192,12 @@ def main():
         if variant == "full":
             a8 = (c(q8), c(k8), c(v8), c(qs), c(ks), c(vs), causal, sm)
             if splits > 1:
+                # a split restarts the running maximum, so its P8 is quantised in another frame than the single pass:
+                # the oracle evaluated with the same split is the reference; the single pass is shown beside it
                 refs["vs_oracle_split_reference_rounding"] = O.attention_full_int8_splitkv(*a8, splits, block_n=bn, out_dtype=dt)
-            refs["vs_reference_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt)
+                refs["vs_single_pass_reference_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt)
+            else:
+                refs["vs_reference_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt)
             if args.p_round == "rne" and splits == 1:
                 refs["vs_same_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt, p_requant=O.p_requant_rne)
         elif variant == "half":
