@@ -560,3 +560,39 @@ def test_other_benchmark_shapes_one_slice_against_oracle(variant, B, H, N, D, ca
                                         p_requant=O.p_requant_rne)
     assert torch.isfinite(o).all()
     assert max_abs(o[b:b + 1, h:h + 1], ref) <= 4e-3 and mean_rel(o[b:b + 1, h:h + 1], ref) <= 2e-4
+
+
+# ------------------------------------------------------------------------------------------ HIP graph capture
+def test_forward_and_quantisers_replay_from_a_captured_graph():
+    """The entry points only enqueue kernels (no allocation, no memset, no synchronisation of their own), so a caller
+    can capture them in a HIP graph: replays interleaved with eager work must reproduce the eager results every time."""
+    g = torch.Generator(device=DEV).manual_seed(80)
+    B, H, N, D = 2, 4, 512, 128
+    x = [torch.randn((B, H, N, D), generator=g, device=DEV, dtype=torch.float16) for _ in range(3)]
+    sm = D ** -0.5
+
+    def pipeline(q, k, v, splits):
+        q8, qs = M.quant_pertoken(q)
+        k8, ks = M.quant_pertoken(k)
+        v8, vs = M.quant_pertensor(v)
+        return M.attention_full_int8(q8, k8, v8, qs, ks, vs, True, sm, num_splits=splits)
+
+    for splits in (1, 3):
+        static = [t.clone() for t in x]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):                       # warm-up outside the capture (library load, allocator pools)
+            pipeline(*static, splits)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = pipeline(*static, splits)
+        for rep in range(4):
+            for t in static:                                # new inputs for every replay, written by eager kernels
+                t.copy_(torch.randn(t.shape, generator=g, device=DEV, dtype=torch.float16))
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = pipeline(*static, splits)
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), (splits, rep)
