@@ -36,9 +36,12 @@ WORKLOADS = {
                                              dtype="bfloat16", std=0.5),
     "full_int8_B16_H16_N1024_d256_bf16": dict(variant="full", B=16, H=16, N=1024, D=256, causal=False, splits=1,
                                               dtype="bfloat16", std=0.5),
+    # the headline shape with V quantised per block of 128 keys and channel (the V scales of the reference's CUDA kernel)
+    "full_int8_B4_H32_N4096_d128_vblock": dict(variant="full", B=4, H=32, N=4096, D=128, causal=False, splits=1, v_block=128),
     # the input quantisers (HBM-bound): Q/K per token, V per (batch, head)
     "quant_pertoken_B4_H32_N4096_d128": dict(variant="quant_token", B=4, H=32, N=4096, D=128, causal=False, splits=1),
     "quant_pertensor_B4_H32_N4096_d128": dict(variant="quant_tensor", B=4, H=32, N=4096, D=128, causal=False, splits=1),
+    "quant_perblock_channel_B4_H32_N4096_d128": dict(variant="quant_block", B=4, H=32, N=4096, D=128, causal=False, splits=1),
 }
 # HBM bytes per launch of the forward kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
 # what the same counter reads for a plain copy of known size; None where not measured.
@@ -80,9 +83,12 @@ def bench_quant(args, variant, x, B, H, N, D, dt):
     reads its input twice (maximum, then quantise)."""
     import torch
     import int_flashattention_amd as M
-    fn = M.quant_pertoken if variant == "quant_token" else M.quant_pertensor
+    fn = {"quant_token": M.quant_pertoken, "quant_tensor": M.quant_pertensor,
+          "quant_block": lambda t: M.quant_perblock_channel(t, 128)}[variant]
     n = B * H * N * D
-    alg_bytes = (2 + 1) * n + (2 * B * H * N if variant == "quant_token" else 2 * B * H) + (2 * n if variant == "quant_tensor" else 0)
+    # (the per-block variant reads its block twice too, but the second sweep of 32 KiB is served by the cache)
+    scale_bytes = {"quant_token": 2 * B * H * N, "quant_tensor": 2 * B * H, "quant_block": 4 * B * H * (N // 128) * D}[variant]
+    alg_bytes = (2 + 1) * n + scale_bytes + (2 * n if variant == "quant_tensor" else 0)
     for _ in range(args.warmup):
         fn(x)
     torch.cuda.synchronize()
@@ -100,7 +106,8 @@ def bench_quant(args, variant, x, B, H, N, D, dt):
            "config": {"workload": args.workload, "batch": B, "heads": H, "seqlen": N, "head_dim": D, "bytes_per_step": alg_bytes},
            "roofline": {"bound": "hbm", "achieved": alg_bytes / (kern_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": alg_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                        "kernel": "quant_pertoken_kernel" if variant == "quant_token" else "quant_slice_amax_kernel + quant_slice_apply_kernel",
+                        "kernel": {"quant_token": "quant_pertoken_kernel", "quant_block": "quant_blockchan_kernel",
+                                   "quant_tensor": "quant_slice_amax_kernel + quant_slice_apply_kernel"}[variant],
                         "avg_launch_ms": kern_ms}}
     print(json.dumps(out))
 
@@ -149,9 +156,10 @@ def main():
         q8, qs = M.quant_pertoken(q)
         k8, ks = M.quant_pertoken(k)
         if variant == "full":
-            v8, vs = M.quant_pertensor(v)
+            v_block = w.get("v_block")
+            v8, vs = M.quant_perblock_channel(v, v_block) if v_block else M.quant_pertensor(v)
             step = lambda: M.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, out_dtype=dt, num_splits=splits,
-                                                 p_round=args.p_round)
+                                                 p_round=args.p_round, v_scale_block=v_block)
         else:
             step = lambda: M.attention_int8(q8, k8, v, qs, ks, causal, sm, num_splits=splits)
     ops = ops_of(B, H, N, D, causal)
@@ -191,15 +199,16 @@ def main():
         refs = {}
         if variant == "full":
             a8 = (c(q8), c(k8), c(v8), c(qs), c(ks), c(vs), causal, sm)
+            okw = dict(v_scale_block=v_block) if v_block else {}
             if splits > 1:
                 # a split restarts the running maximum, so its P8 is quantised in another frame than the single pass:
                 # the oracle evaluated with the same split is the reference; the single pass is shown beside it
                 refs["vs_oracle_split_reference_rounding"] = O.attention_full_int8_splitkv(*a8, splits, block_n=bn, out_dtype=dt)
                 refs["vs_single_pass_reference_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt)
             else:
-                refs["vs_reference_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt)
+                refs["vs_reference_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt, **okw)
             if args.p_round == "rne" and splits == 1:
-                refs["vs_same_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt, p_requant=O.p_requant_rne)
+                refs["vs_same_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt, p_requant=O.p_requant_rne, **okw)
         elif variant == "half":
             refs["vs_oracle"] = O.attention_int8(c(q8), c(k8), c(v), c(qs), c(ks), causal, sm, block_n=bn, out_dtype=dt)
         else:
@@ -231,7 +240,8 @@ def main():
                    "inputs": f"Q,K,V {str(dt).replace('torch.', '')} ~ N(0,{std}), seed 20"
                              + (f", K channels {outlier_cols} x20" if outlier_cols else "")
                              + ("; Q,K per-token int8" if variant != "fp" else "")
-                             + (", V per-(batch,head) int8" if variant == "full" else "")},
+                             + ((f", V int8 per block of {w['v_block']} keys and channel" if w.get("v_block")
+                                 else ", V per-(batch,head) int8") if variant == "full" else "")},
         "pct_int8_peak": 100.0 * value / INT8_PEAK_TOPS,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TOP/s" if variant == "full" else "TFLOP/s",
                      "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),

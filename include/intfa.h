@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define INTFA_VERSION 2
+#define INTFA_VERSION 3
 
 /* forward variants (one entry point each, below) */
 enum { INTFA_VARIANT_FULL_INT8 = 0, INTFA_VARIANT_HALF_INT8 = 1, INTFA_VARIANT_FP16 = 2 };
@@ -55,7 +55,8 @@ enum {
     INTFA_ERR_WORKSPACE = -6,     /* workspace missing or too small for the requested split count */
     INTFA_ERR_SHAPE = -7,         /* batch/heads not positive, a row stride below head_dim, a (batch, head) slice of
                                      k or v spanning 4 GiB or more, or sizes that overflow 32-bit block indices */
-    INTFA_ERR_SPLITS = -8         /* num_splits out of range */
+    INTFA_ERR_SPLITS = -8,        /* num_splits out of range */
+    INTFA_ERR_VSCALE = -9         /* v_scale_block not a multiple of the key-block length, or vs_stride_blk below head_dim */
 };
 
 /*
@@ -75,7 +76,8 @@ typedef struct intfa_fwd_params {
     void*       out;
     const void* q_scale;      /* [batch, heads, seqlen], scale_dtype */
     const void* k_scale;      /* [batch, heads, seqlen], scale_dtype */
-    const void* v_scale;      /* [batch, heads], scale_dtype */
+    const void* v_scale;      /* [batch, heads], scale_dtype; with v_scale_block set:
+                                 [batch, heads, ceil(seqlen_k / v_scale_block), head_dim], always fp32 */
     float*      lse;          /* optional [batch, heads, seqlen] contiguous: m + log2(l), base-2 as the
                                  reference's M (flash_atten_int8.py:172-175); NULL = not written */
 
@@ -107,6 +109,16 @@ typedef struct intfa_fwd_params {
     int32_t seqlen_k;         /* number of keys when it differs from the number of queries (cross attention, decoding
                                  against a cache): k, v and k_scale then have seqlen_k rows.  0 = seqlen.  Not with
                                  causal (the reference's mask is defined for equal lengths). */
+    int32_t v_scale_block;    /* full-int8 only.  0: one V scale per (batch, head), the reference's Python API
+                                 (flash_atten_full_int8.py:159-161).  > 0: V was quantised per block of v_scale_block keys
+                                 and per channel, the layout its CUDA kernel reads (csrc/flash_fwd_kernel_full_qi8.h:
+                                 156-160, applied per key block at csrc/mask.h:313-340); v_scale then has one row of
+                                 head_dim fp32 scales per block of keys (channel stride 1, row stride vs_stride_blk, batch
+                                 and head strides vs_stride_b / vs_stride_h over heads_kv heads; 4-byte aligned, fp32 as in
+                                 that kernel whatever scale_dtype says).  Must be a multiple of
+                                 intfa_fwd_block_n(INTFA_VARIANT_FULL_INT8, head_dim). */
+    int32_t reserved0;        /* set to 0 */
+    int64_t vs_stride_blk;    /* elements between consecutive scale rows of v_scale (>= head_dim) */
 } intfa_fwd_params;
 
 /* Library/ABI version (INTFA_VERSION of the build). */
@@ -146,9 +158,8 @@ int intfa_fwd_half_int8(const intfa_fwd_params* p, void* stream);
 int intfa_fwd_fp16(const intfa_fwd_params* p, void* stream);
 
 /* Debug export of the int32 accumulators S = Q8 K8^T produced by the same MFMA tile code the forward
- * uses (flash_atten_full_int8.py:36).  s_out is [batch, heads, seqlen, seqlen] int32, contiguous.
- * s_out is [batch, heads, seqlen, seqlen_k].  Uses q, k and their strides, batch, heads, seqlen, seqlen_k, head_dim
- * of the block. */
+ * uses (flash_atten_full_int8.py:36).  s_out is [batch, heads, seqlen, seqlen_k] int32, contiguous.  Uses q, k and
+ * their strides, batch, heads, heads_kv, seqlen, seqlen_k and head_dim of the block. */
 int intfa_debug_qk_int32(const intfa_fwd_params* p, int32_t* s_out, void* stream);
 
 /* quant_pertoken(X) -> (int8 X, scale) of the reference's harness (benchmark.py:96-100): per row of head_dim
@@ -166,6 +177,16 @@ size_t intfa_quant_pertensor_workspace_bytes(int32_t batch, int32_t heads);
 int intfa_quant_pertensor(const void* x, int64_t stride_b, int64_t stride_h, int64_t stride_n, void* q8, void* scale,
                           int32_t batch, int32_t heads, int32_t seqlen, int32_t head_dim, int32_t dtype,
                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* Quantiser for the blocked V scales of intfa_fwd_params.v_scale_block: one fp32 scale per (batch, head, block of
+ * `block` rows, channel), scale = absmax / 127 over the block's rows and q = round-half-even(x / scale), both in fp32
+ * (the harness's formula, benchmark.py:102-107, at the granularity of the V scales its CUDA kernel reads,
+ * csrc/flash_fwd_kernel_full_qi8.h:156-160; the reference itself holds no quantiser for that layout).  A channel that
+ * is zero throughout a block gets scale 0 and zeros.  x as for intfa_quant_pertoken; q8 int8 contiguous; scale fp32
+ * [batch, heads, ceil(seqlen / block), head_dim] contiguous, 16-byte aligned. */
+int intfa_quant_perblock_channel(const void* x, int64_t stride_b, int64_t stride_h, int64_t stride_n, void* q8, float* scale,
+                                 int32_t batch, int32_t heads, int32_t seqlen, int32_t head_dim, int32_t block,
+                                 int32_t dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libintfa.so")
 
-ABI_VERSION = 2          # INTFA_VERSION of include/intfa.h this mirror was written against
+ABI_VERSION = 3          # INTFA_VERSION of include/intfa.h this mirror was written against
 INTFA_F16, INTFA_BF16, INTFA_F32 = 0, 1, 2
 PROUND_RNE, PROUND_REFERENCE = 0, 1
 
@@ -31,7 +31,8 @@ class FwdParams(ctypes.Structure):
         + [(n, ctypes.c_int32) for n in ("batch", "heads", "seqlen", "head_dim", "scale_dtype", "io_dtype", "causal")]
         + [("sm_scale", ctypes.c_float), ("p_round", ctypes.c_int32), ("num_splits", ctypes.c_int32),
            ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
-           ("heads_kv", ctypes.c_int32), ("seqlen_k", ctypes.c_int32)]
+           ("heads_kv", ctypes.c_int32), ("seqlen_k", ctypes.c_int32),
+           ("v_scale_block", ctypes.c_int32), ("reserved0", ctypes.c_int32), ("vs_stride_blk", ctypes.c_int64)]
     )
 
 
@@ -39,7 +40,8 @@ VARIANT_FULL_INT8, VARIANT_HALF_INT8, VARIANT_FP16 = 0, 1, 2
 
 EXPORTS = ("intfa_version", "intfa_error_string", "intfa_fwd_block_n", "intfa_fwd_workspace_bytes", "intfa_fwd_suggest_splits",
            "intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16", "intfa_debug_qk_int32",
-           "intfa_quant_pertoken", "intfa_quant_pertensor_workspace_bytes", "intfa_quant_pertensor")
+           "intfa_quant_pertoken", "intfa_quant_pertensor_workspace_bytes", "intfa_quant_pertensor",
+           "intfa_quant_perblock_channel")
 
 _lib = None
 
@@ -78,6 +80,8 @@ def load():
     lib.intfa_quant_pertensor_workspace_bytes.argtypes = [i32, i32]
     lib.intfa_quant_pertensor.restype = ctypes.c_int
     lib.intfa_quant_pertensor.argtypes = [vp, i64, i64, i64, vp, vp, i32, i32, i32, i32, i32, vp, ctypes.c_size_t, vp]
+    lib.intfa_quant_perblock_channel.restype = ctypes.c_int
+    lib.intfa_quant_perblock_channel.argtypes = [vp, i64, i64, i64, vp, vp, i32, i32, i32, i32, i32, i32, vp]
     if lib.intfa_version() != ABI_VERSION:
         raise RuntimeError(f"{LIB_PATH} has ABI version {lib.intfa_version()}, this package expects {ABI_VERSION}: rebuild it")
     _lib = lib

@@ -55,7 +55,8 @@ def _require_gpu(*ts):
 
 
 def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float, out_dtype,
-                   num_splits: int = 1, p_round: int = _capi.PROUND_RNE, return_lse: bool = False):
+                   num_splits: int = 1, p_round: int = _capi.PROUND_RNE, return_lse: bool = False,
+                   v_scale_block: Optional[int] = None):
     lib = _capi.load()
     _require_gpu(q, k, v, q_scale, k_scale, v_scale)
     d = check_head_dims(q, k, v)
@@ -92,9 +93,23 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
         p.ks_stride_b, p.ks_stride_h, p.ks_stride_n = k_scale.stride()
         keep += [q_scale, k_scale]
     if variant == "full":
-        vs = v_scale if v_scale.dtype == q_scale.dtype else v_scale.to(q_scale.dtype)
+        if v_scale.dim() == 4:
+            vs = v_scale.float()                                     # blocked scales cross the ABI as fp32
+            # one scale per block of keys and channel ([Z, H_kv, ceil(N_k / v_scale_block), d])
+            vsb = block_n("full", d) if v_scale_block is None else int(v_scale_block)
+            if vsb <= 0 or tuple(vs.shape) != (Z, H_kv, (N_k + vsb - 1) // vsb, d):
+                raise ValueError(f"a blocked v_scale must be [Z, H_kv, ceil(N_k / {vsb}), d], got {tuple(vs.shape)}")
+            vs = _pad_head_dim(vs, dk)
+            if vs.stride(-1) != 1:
+                vs = vs.contiguous()
+            p.v_scale_block = vsb
+            p.vs_stride_b, p.vs_stride_h, p.vs_stride_blk = vs.stride()[:3]
+        else:
+            if v_scale_block is not None:
+                raise ValueError("v_scale_block needs a 4-D v_scale")
+            vs = v_scale if v_scale.dtype == q_scale.dtype else v_scale.to(q_scale.dtype)
+            p.vs_stride_b, p.vs_stride_h = vs.stride()
         p.v_scale = vs.data_ptr()
-        p.vs_stride_b, p.vs_stride_h = vs.stride()
         keep.append(vs)
     p.batch, p.heads, p.seqlen, p.head_dim = Z, H, N, dk
     p.heads_kv = H_kv

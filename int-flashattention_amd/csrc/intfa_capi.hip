@@ -14,6 +14,13 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 int scale_size(int dt) { return dt == INTFA_F32 ? 4 : 2; }
 
+// Key-block length of a variant at a head_dim: the full-int8 kernel takes 128 keys per block (64 at head_dim 256),
+// the kernels with a 16-bit P V take 64.
+int block_n_for(int variant, int head_dim) {
+    if (variant == INTFA_VARIANT_FULL_INT8) return head_dim <= 128 ? 128 : 64;
+    return 64;
+}
+
 // Common validation; fills the kernel-side block.  elem sizes in bytes for q/k, v and out.
 int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need_scales, bool need_vscale, KParams* kp) {
     if (p == nullptr || p->q == nullptr || p->k == nullptr) return INTFA_ERR_NULL;
@@ -59,6 +66,14 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
     if (need_vscale) {
         if (p->v_scale == nullptr) return INTFA_ERR_NULL;
         k.v_scale = (const char*)p->v_scale; k.vs_sb = p->vs_stride_b; k.vs_sh = p->vs_stride_h;
+        if (p->v_scale_block < 0) return INTFA_ERR_VSCALE;
+        if (p->v_scale_block > 0) {
+            const int bn = block_n_for(INTFA_VARIANT_FULL_INT8, p->head_dim);
+            if (p->v_scale_block % bn != 0 || p->vs_stride_blk < p->head_dim) return INTFA_ERR_VSCALE;
+            if (reinterpret_cast<uintptr_t>(p->v_scale) & 3u) return INTFA_ERR_ALIGN;
+            k.vs_g = p->v_scale_block / bn;
+            k.vs_sblk = p->vs_stride_blk;
+        }
     }
     k.lse = p->lse;
     k.batch = p->batch; k.heads = p->heads; k.seqlen = p->seqlen; k.seqlen_k = seqlen_k; k.head_dim = p->head_dim;
@@ -103,14 +118,8 @@ int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t str
     return e == hipSuccess ? INTFA_OK : (int)e;
 }
 
-// Key-block length of a variant at a head_dim: the full-int8 kernel takes 128 keys per block (64 at head_dim 256),
-// the kernels with a 16-bit P V take 64.
-int block_n_for(int variant, int head_dim) {
-    if (variant == INTFA_VARIANT_FULL_INT8) return head_dim <= 128 ? 128 : 64;
-    return 64;
-}
-
 int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dump_s, hipStream_t stream) {
+    const bool vblk = variant == INTFA_VARIANT_FULL_INT8 && !dump_s && kp.vs_g > 0;
     LaunchSel sel;
     sel.causal = kp.causal != 0;
     sel.io_dt = p->io_dtype == INTFA_BF16 ? 1 : 0;
@@ -118,7 +127,11 @@ int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dum
     sel.split = kp.num_splits > 1;
     sel.dump_s = dump_s;
     const int d = kp.head_dim;
-    if (variant == INTFA_VARIANT_FULL_INT8) {
+    if (vblk) {
+        if (d == 64) return launch_full_int8_vblk_d64(kp, sel, stream);
+        if (d == 128) return launch_full_int8_vblk_d128(kp, sel, stream);
+        if (d == 256) return launch_full_int8_vblk_d256(kp, sel, stream);
+    } else if (variant == INTFA_VARIANT_FULL_INT8) {
         if (d == 64) return launch_full_int8_d64(kp, sel, stream);
         if (d == 128) return launch_full_int8_d128(kp, sel, stream);
         if (d == 256) return launch_full_int8_d256(kp, sel, stream);
@@ -170,6 +183,7 @@ const char* intfa_error_string(int code) {
         case INTFA_ERR_WORKSPACE: return "workspace missing, misaligned or too small for num_splits";
         case INTFA_ERR_SHAPE: return "batch and heads must be positive and the grid must fit 31 bits";
         case INTFA_ERR_SPLITS: return "num_splits must be at most 64";
+        case INTFA_ERR_VSCALE: return "v_scale_block must be a multiple of the key-block length and vs_stride_blk at least head_dim";
         default: return code > 0 ? "hip error" : "unknown error";
     }
 }

@@ -52,11 +52,13 @@ struct KParams {
     int64_t qs_sb, qs_sh, qs_sn;           // elements
     int64_t ks_sb, ks_sh, ks_sn;
     int64_t vs_sb, vs_sh;
+    int64_t vs_sblk;                       // blocked V scales: elements between the scale rows of consecutive key ranges
     int32_t batch, heads, seqlen, head_dim;  // seqlen = number of query rows
     int32_t seqlen_k;                      // number of keys (= seqlen unless the caller passes separate lengths)
     int32_t scale_dtype, causal, num_splits, blocks_per_split;
     int32_t kv_group;                      // query heads per K/V head (1 = every query head has its own K/V)
     int32_t pair_mblocks;                  // causal single-pass launches: one workgroup takes query blocks i and n-1-i
+    int32_t vs_g;                          // blocked V scales: key blocks of the kernel per scale row (0 = scalar V scale)
     float qk_scale_log2;                   // sm_scale * log2(e)
 };
 

@@ -29,7 +29,10 @@ template <int D> struct FullInt8Geom {
     static constexpr int NHALF = D / DV;
 };
 
-template <int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUMP_S, bool SPLIT>
+// VBLK: V carries one scale per key block and channel (layout of the reference's CUDA kernel,
+// csrc/flash_fwd_kernel_full_qi8.h:156-160) instead of one per (batch, head): the int32 P V of a block is multiplied
+// by the block's channel scales before it joins the accumulator (csrc/mask.h:313-340).
+template <int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUMP_S, bool SPLIT, bool VBLK = false>
 __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T (32 bytes of head_dim each)
@@ -48,7 +51,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     constexpr int OFF_KS = 0;                    // two fp32 k_scale vectors
     constexpr int OFF_K = 2 * BN * 4;            // two K tiles
     constexpr int OFF_V = OFF_K + 2 * KT;        // two V tiles
-    constexpr int LDS_BYTES = OFF_V + 2 * VT;
+    constexpr int OFF_VS = OFF_V + 2 * VT;       // VBLK: two vectors of DV fp32 channel scales
+    constexpr int LDS_BYTES = OFF_VS + (VBLK ? 2 * DV * 4 : 0);
     __shared__ __attribute__((aligned(1024))) char smem[LDS_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -182,6 +186,19 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         if (p.scale_dtype == 1) return __builtin_bit_cast(float, raw << 16);
         return __builtin_bit_cast(float, raw);
     };
+    // VBLK: channel scales of a key block; thread 128 + c fetches the scale of this workgroup's channel c.  A scale
+    // row covers vs_g key blocks.
+    const int vs_c = tid - 128;
+    const bool vs_thread = VBLK && vs_c >= 0 && vs_c < DV;
+    // (these scales are fp32 whatever the type of the per-token scales, as in the reference's kernel)
+    const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + half * DV + (vs_thread ? vs_c : 0));
+    auto load_vs = [&](int nb) __attribute__((always_inline)) -> float {
+        if (!VBLK) return 0.f;
+        const int row = p.vs_g == 1 ? nb : nb / p.vs_g;
+        return Vsg[(int64_t)row * p.vs_sblk];
+    };
+    const uint32_t vs_wr = OFF_VS + 4 * (vs_thread ? vs_c : 0);
+    const uint32_t vs_rd = OFF_VS + 16 * lh;       // + 4 * (32*dt + 8*a4) per read
 
     // ---- per-lane LDS read offsets (everything else is an immediate)
     // K (A operand of S^T): lane reads row (32*st + lq), chunk (2*ks + lh), XOR-swizzled by the row
@@ -359,6 +376,13 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         // -------- P V on int8 MFMA: O^T[d, q] += V^T[d, key] P^T[key, q]; the chain of d-tile dt+1 is issued
         // before the accumulator update of d-tile dt, its V fragments were requested two stages earlier.
         v16i oacc[2];
+        constexpr int VSB = BUF * DV * 4;
+        v4f vsc[2][4];                          // VBLK: channel scales of the d-tile being folded in / the next one
+        auto load_vsc = [&](v4f (&dst)[4], int dt) __attribute__((always_inline)) {
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4) dst[a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (32 * dt + 8 * a4));
+        };
+        if (VBLK) load_vsc(vsc[0], 0);
         auto pv_chain = [&](v16i& acc, const v4i (&f)[NST]) __attribute__((always_inline)) {
             acc = (v16i){0};
 #pragma unroll
@@ -375,6 +399,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         for (int dt = 0; dt < DT; ++dt) {
             __builtin_amdgcn_sched_barrier(0);
             if (dt + 2 < DT) load_vfrags(vf[dt & 1], dt + 2);
+            if (VBLK && dt + 1 < DT) load_vsc(vsc[(dt + 1) & 1], dt + 1);
             v16i& nacc = oacc[(dt + 1) & 1];
 #pragma unroll
             for (int a4 = 0; a4 < 4; ++a4) {
@@ -391,7 +416,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
 #pragma unroll
                 for (int b4 = 0; b4 < 4; ++b4) {
                     const int r = 4 * a4 + b4;
-                    o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, (float)oacc[dt & 1][r]);
+                    if (VBLK) o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, (float)oacc[dt & 1][r] * vsc[dt & 1][a4][b4]);
+                    else o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, (float)oacc[dt & 1][r]);
                     asm volatile("" : "+v"(o_acc[dt][r]));     // keeps the update in this slot (it would be sunk below the loop)
                 }
             }
@@ -407,13 +433,16 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         __syncthreads();
         const bool more = nb + 1 < nb_end;
         uint32_t ks_next = 0;
+        float vs_next = 0.f;
         constexpr bool DIAG = decltype(diag_tag)::value;
         if (more) {
             if (DUMP_S || DIAG) issue_loads(nb + 1, BUF ^ 1);      // (a diagonal block is the last one: more == false)
             ks_next = load_ks(nb + 1);
+            if (vs_thread) vs_next = load_vs(nb + 1);
         }
         compute(buf_tag, diag_tag, nb, more, gw, lim);
         if (more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
+        if (more && vs_thread) *(float*)(smem + vs_wr + (BUF ^ 1) * DV * 4) = vs_next;
     };
 
     // ---- main loop: K/V tiles double-buffered in LDS, one barrier per key block.  The block on the causal
@@ -423,6 +452,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         {
             const uint32_t s0 = load_ks(nb_begin);
             if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
+            if (vs_thread) *(float*)(smem + vs_wr) = load_vs(nb_begin);
         }
         const int diag_begin = mb * RDIAG;                 // first key block that touches the diagonal
         const int tail_keys = p.seqlen_k - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
@@ -456,7 +486,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     const int e_heads = pe->heads, e_seqlen = pe->seqlen;
     const int eb = head / e_heads, eh = head % e_heads;
     const float l_tot = half_pair_sum(l_run);          // in units of 1/127 when PROUND == 0
-    const float vs = load_scale(pe->v_scale, eb * pe->vs_sb + (eh / pe->kv_group) * pe->vs_sh, pe->scale_dtype);
+    const float vs = VBLK ? 1.f : load_scale(pe->v_scale, eb * pe->vs_sb + (eh / pe->kv_group) * pe->vs_sh, pe->scale_dtype);
     const float out_scale = (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
     const float l_true = (PROUND == 0) ? l_tot * (1.f / 127.f) : l_tot;
     const float lse = m_run + __builtin_log2f(l_true);

@@ -25,6 +25,9 @@ template <typename K> inline int launch_kernel(K kernel, const KParams& kp, hipS
 INTFA_DECL_LAUNCH(launch_full_int8_d64);
 INTFA_DECL_LAUNCH(launch_full_int8_d128);
 INTFA_DECL_LAUNCH(launch_full_int8_d256);
+INTFA_DECL_LAUNCH(launch_full_int8_vblk_d64);     // per-block, per-channel V scales
+INTFA_DECL_LAUNCH(launch_full_int8_vblk_d128);
+INTFA_DECL_LAUNCH(launch_full_int8_vblk_d256);
 INTFA_DECL_LAUNCH(launch_half_int8_d64);
 INTFA_DECL_LAUNCH(launch_half_int8_d128);
 INTFA_DECL_LAUNCH(launch_half_int8_d256);

@@ -178,6 +178,79 @@ template <int DT, int LPR> __global__ void __launch_bounds__(256) quant_slice_ap
     }
 }
 
+// ---- per (batch, head, block of rows, channel): fp32 scales, the layout of the V scales of the reference's CUDA
+// kernel (csrc/flash_fwd_kernel_full_qi8.h:156-160).  One workgroup owns one block of rows: column maxima through LDS
+// atomics, then a second sweep over the block (served by the cache) that divides and rounds in fp32.
+template <int DT, int LPR> __global__ void __launch_bounds__(256) quant_blockchan_kernel(const QuantParams p, int block, int nblk,
+                                                                                         float* scale_out) {
+    constexpr int RPB = 256 / LPR;
+    __shared__ uint32_t smax[LPR * 8];
+    const int sub = threadIdx.x % LPR, rl = threadIdx.x / LPR;
+    const int bh = blockIdx.x / nblk, blk = blockIdx.x % nblk;
+    const int64_t h = bh % p.heads, b = bh / p.heads;
+    const int n_lo = blk * block, n_hi = n_lo + block < p.seqlen ? n_lo + block : p.seqlen;
+    const char* base = p.x + b * p.sb + h * p.sh + sub * 16;
+    for (int i = threadIdx.x; i < LPR * 8; i += 256) smax[i] = 0u;
+    __syncthreads();
+    uint32_t m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int n0 = n_lo + rl; n0 < n_hi; n0 += RPB * kRowsInFlight) {
+        v4i raw[kRowsInFlight];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const int n = n0 + u * RPB;
+            raw[u] = n < n_hi ? *(const v4i*)(base + (int64_t)n * p.sn) : (v4i){0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t w = (uint32_t)raw[u][j / 2];
+                const uint32_t a = abs_bits((uint16_t)(j & 1 ? w >> 16 : w & 0xffffu));
+                m[j] = m[j] > a ? m[j] : a;
+            }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) atomicMax(&smax[sub * 8 + j], m[j]);
+    __syncthreads();
+    float sc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sc[j] = to_f32<DT>((uint16_t)smax[sub * 8 + j]) / 127.0f;
+    if (rl == 0) {
+        float* dst = scale_out + ((int64_t)bh * nblk + blk) * p.head_dim + sub * 8;
+        *(v4f*)dst = (v4f){sc[0], sc[1], sc[2], sc[3]};
+        *(v4f*)(dst + 4) = (v4f){sc[4], sc[5], sc[6], sc[7]};
+    }
+    char* qbase = p.q8 + (int64_t)bh * p.seqlen * p.head_dim + sub * 8;
+    for (int n0 = n_lo + rl; n0 < n_hi; n0 += RPB * kRowsInFlight) {
+        v4i raw[kRowsInFlight];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const int n = n0 + u * RPB;
+            raw[u] = n < n_hi ? *(const v4i*)(base + (int64_t)n * p.sn) : (v4i){0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const int n = n0 + u * RPB;
+            if (n >= n_hi) continue;
+            int out[2];
+#pragma unroll
+            for (int w2 = 0; w2 < 2; ++w2) {
+                uint32_t pk = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t word = (uint32_t)raw[u][2 * w2 + j / 2];
+                    const float x = to_f32<DT>((uint16_t)(j & 1 ? word >> 16 : word & 0xffffu));
+                    const float s = sc[4 * w2 + j];
+                    const int q = s > 0.f ? (int)__builtin_rintf(x / s) : 0;        // IEEE division, round-half-even
+                    pk |= ((uint32_t)q & 0xffu) << (8 * j);
+                }
+                out[w2] = (int)pk;
+            }
+            *(v2i*)(qbase + (int64_t)n * p.head_dim) = (v2i){out[0], out[1]};
+        }
+    }
+}
+
 int check(const void* x, const void* q8, const void* scale, int64_t sb, int64_t sh, int64_t sn, int batch, int heads,
           int seqlen, int head_dim, int dtype, QuantParams* qp) {
     if (x == nullptr || q8 == nullptr || scale == nullptr) return INTFA_ERR_NULL;
@@ -253,6 +326,26 @@ int intfa_quant_pertensor(const void* x, int64_t stride_b, int64_t stride_h, int
         const int g = grid_for(qp.rows, rpb); \
         if (dtype == INTFA_F16) hipLaunchKernelGGL((quant_slice_apply_kernel<0, LPR>), dim3(g), dim3(256), 0, st, qp); \
         else hipLaunchKernelGGL((quant_slice_apply_kernel<1, LPR>), dim3(g), dim3(256), 0, st, qp); } while (0)
+    INTFA_LPR_SWITCH(head_dim, INTFA_CALL)
+#undef INTFA_CALL
+    return (int)hipGetLastError();
+}
+
+int intfa_quant_perblock_channel(const void* x, int64_t stride_b, int64_t stride_h, int64_t stride_n, void* q8, float* scale,
+                                 int32_t batch, int32_t heads, int32_t seqlen, int32_t head_dim, int32_t block,
+                                 int32_t dtype, void* stream) {
+    QuantParams qp;
+    const int rc = check(x, q8, scale, stride_b, stride_h, stride_n, batch, heads, seqlen, head_dim, dtype, &qp);
+    if (rc != INTFA_OK) return rc;
+    if (block <= 0) return INTFA_ERR_VSCALE;
+    if (reinterpret_cast<uintptr_t>(scale) & 15u) return INTFA_ERR_ALIGN;
+    const int nblk = (seqlen + block - 1) / block;
+    const int64_t grid = (int64_t)batch * heads * nblk;
+    if (grid >= (1ll << 31)) return INTFA_ERR_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+#define INTFA_CALL(LPR) do { \
+        if (dtype == INTFA_F16) hipLaunchKernelGGL((quant_blockchan_kernel<0, LPR>), dim3((int)grid), dim3(256), 0, st, qp, block, nblk, scale); \
+        else hipLaunchKernelGGL((quant_blockchan_kernel<1, LPR>), dim3((int)grid), dim3(256), 0, st, qp, block, nblk, scale); } while (0)
     INTFA_LPR_SWITCH(head_dim, INTFA_CALL)
 #undef INTFA_CALL
     return (int)hipGetLastError();

@@ -6,7 +6,7 @@ from ._host import launch_forward
 
 
 def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, *, out_dtype=torch.float16,
-                        num_splits=1, p_round="rne", return_lse=False):
+                        num_splits=1, p_round="rne", return_lse=False, v_scale_block=None):
     """Full-int8 attention forward.
 
     q, k, v: int8 [Z, H, N, d]; q_scale, k_scale: [Z, H, N] per-token scales; v_scale: [Z, H];
@@ -15,9 +15,14 @@ def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, *,
     the off-diagonal and diagonal stages (as flash_atten_int8.py:157-166 does), not the reference's
     full-int8 behaviour, which restarts from -inf (flash_atten_full_int8.py:166,175).
 
+    ``v_scale`` may also be 4-D, [Z, H, ceil(N / v_scale_block), d]: one scale per block of ``v_scale_block`` keys and
+    channel, the V scales of the reference's CUDA kernel (csrc/flash_fwd_kernel_full_qi8.h:156-160), as produced by
+    ``quant_perblock_channel``.  ``v_scale_block`` defaults to the kernel's key-block length (``block_n("full", d)``)
+    and must be a multiple of it.
+
     ``p_round``: "rne" folds 127 into the exponent and rounds to nearest-even; "reference" reproduces the
     fp16 sequence of flash_atten_full_int8.py:49-51.
     """
     pr = {"rne": _capi.PROUND_RNE, "reference": _capi.PROUND_REFERENCE}[p_round]
     return launch_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, out_dtype,
-                          num_splits=num_splits, p_round=pr, return_lse=return_lse)
+                          num_splits=num_splits, p_round=pr, return_lse=return_lse, v_scale_block=v_scale_block)

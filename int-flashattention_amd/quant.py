@@ -54,3 +54,25 @@ def quant_pertensor(x):
     for t in (x_, ws):
         t.record_stream(torch.cuda.current_stream(x.device))
     return q8, scale
+
+
+def quant_perblock_channel(x, block):
+    """One fp32 scale per (batch, head, block of ``block`` rows, channel) - the layout of the V scales that the
+    reference's CUDA kernel reads (csrc/flash_fwd_kernel_full_qi8.h:156-160) - with the harness's formula
+    (benchmark.py:102-107: absmax / 127, round-half-even) evaluated in fp32.  Returns (int8 [Z,H,N,d], fp32
+    [Z,H,ceil(N/block),d]); pass both to ``attention_full_int8(..., v_scale_block=block)``."""
+    lib = _capi.load()
+    x_ = _prepare(x)
+    Z, H, N, d = x_.shape
+    block = int(block)
+    if block <= 0:
+        raise ValueError("block must be positive")
+    q8 = torch.empty((Z, H, N, d), dtype=torch.int8, device=x.device)
+    scale = torch.empty((Z, H, (N + block - 1) // block, d), dtype=torch.float32, device=x.device)
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    with torch.cuda.device(x.device):
+        rc = lib.intfa_quant_perblock_channel(x_.data_ptr(), x_.stride(0), x_.stride(1), x_.stride(2), q8.data_ptr(),
+                                              scale.data_ptr(), Z, H, N, d, block, _DT[x.dtype], ctypes.c_void_p(stream))
+    _capi.check(rc, "intfa_quant_perblock_channel")
+    x_.record_stream(torch.cuda.current_stream(x.device))
+    return q8, scale

@@ -17,6 +17,12 @@ What each function follows in the reference (paths relative to the reference che
                                  full-int8 file drops it (flash_atten_full_int8.py:71,166,175 return only acc, l_i)
 * ``attention_int8``           - flash_atten_int8.py:9-66, :140-176 (also returns M = m + log2(l), :172-175)
 * ``attention_fp``             - flash_atten_fp.py:9-60, :115-150
+* ``quant_perblock_channel``   - no quantiser for this layout exists in the reference; it applies the harness's formula
+                                 (benchmark.py:102-107: absmax / 127, round-half-even) at the granularity of the V scale
+                                 tensor its CUDA kernel reads (csrc/flash_fwd_kernel_full_qi8.h:156-160: one fp32 scale
+                                 per key block and channel)
+* ``attention_full_int8`` with a 4-D ``v_scale`` - the per-block, per-channel dequantisation of P V of that kernel
+                                 (csrc/mask.h:313-340: acc_o += scale_col[col] * acc_o_int / 127)
 * ``splitkv_ranges``           - csrc/flash_fwd_kernel.h:503-511 (key-block range of a split)
 * ``splitkv_combine``          - csrc/flash_fwd_kernel.h:1212-1235 (log-sum-exp over splits), :1264-1283 (weighted sum)
 
@@ -35,6 +41,9 @@ How every function is pinned (tests/test_oracle.py):
   is that constant times sum(P8)/(127 l).
 * causal: equality with a dense tril-masked evaluation; first row attends to key 0 only.
 * split-KV: any split count agrees with one split to fp32 rounding.
+* blocked V scales: a 4-D scale tensor filled with one value per (batch, head) reproduces the scalar form bit for
+  bit; the result equals the scalar form applied to V pre-multiplied by the block/channel factors when these are
+  powers of two; ``quant_perblock_channel`` against a pure-Python loop, and every (block, channel) reaches +-127.
 
 The reference holds no golden vectors for this path (its only test asserts the fp16 forward with
 atol=1e-2, benchmark.py:242), so none are used.
@@ -67,6 +76,24 @@ def quant_pertensor(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     x_scale = x_max / 127
     ret = torch.round(x / x_scale[:, :, None, None]).to(torch.int8)
     return ret, x_scale
+
+
+def quant_perblock_channel(x: torch.Tensor, block: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One fp32 scale per (batch, head, block of ``block`` rows, channel): scale = absmax / 127 over the block's rows,
+    int8 = round-half-even(x / scale), both in fp32.  Returns (int8 [B,H,N,d], scale [B,H,ceil(N/block),d]).  A channel
+    that is all zero inside a block gets scale 0 and int8 0."""
+    B, H, N, D = x.shape
+    nblk = (N + block - 1) // block
+    xf = x.float()
+    pad = nblk * block - N
+    if pad:
+        xf = torch.cat([xf, torch.zeros((B, H, pad, D))], dim=2)
+    xb = xf.view(B, H, nblk, block, D)
+    scale = xb.abs().amax(dim=3) / 127                                       # [B,H,nblk,D] fp32
+    safe = torch.where(scale > 0, scale, torch.ones_like(scale))
+    q = torch.round(xb / safe[:, :, :, None, :])
+    q = torch.where(scale[:, :, :, None, :] > 0, q, torch.zeros_like(q))
+    return q.view(B, H, nblk * block, D)[:, :, :N].to(torch.int8).contiguous(), scale
 
 
 def mean_relative_error(a: torch.Tensor, b: torch.Tensor, calc_num: Optional[int] = None) -> float:
@@ -138,13 +165,15 @@ def p_requant_rne(p: torch.Tensor) -> torch.Tensor:
 def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float,
                      block_m: int, block_n: int, key_lo: int = 0, key_hi: Optional[int] = None,
                      p_requant=p_requant_reference, pv_dtype=torch.float16,
-                     row_lo: int = 0, row_hi: Optional[int] = None):
+                     row_lo: int = 0, row_hi: Optional[int] = None, v_scale_block: Optional[int] = None):
     """Runs the reference's tile loop over key blocks [key_lo, key_hi) for every query row at once.
 
     Rows are grouped in tiles of ``block_m`` as the reference's programs are; for a causal run a tile sees
     the key blocks below its first row without a mask (stage 1) and the blocks of its own row range with the
     mask (stage 2), flash_atten_full_int8.py:18-25.  Returns fp32 (acc, l, m) with acc un-normalised.
     Only rows [row_lo, row_hi) are evaluated (the others keep m = -inf, l = 1, acc = 0).
+    A 4-D ``v_scale`` [B,H,ceil(N/v_scale_block),d] selects the per-block, per-channel dequantisation of P V
+    (csrc/mask.h:313-340); ``v_scale_block`` must be a multiple of ``block_n``.
     """
     B, H, N, D = q.shape
     key_hi = N if key_hi is None else key_hi
@@ -162,7 +191,11 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
     if int_qk:
         qs = q_scale.float()
         ks = k_scale.float()
-    if variant == "full":
+    vs_blocked = variant == "full" and v_scale.dim() == 4
+    if vs_blocked:
+        v_scale_block = block_n if v_scale_block is None else v_scale_block
+        assert v_scale_block % block_n == 0 and v_scale.shape[2] == (k.shape[2] + v_scale_block - 1) // v_scale_block
+    elif variant == "full":
         vs = v_scale.float()[:, :, None, None]
     rows = torch.arange(N)
 
@@ -202,6 +235,8 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
             if variant == "full":
                 p8 = p_requant(p)                                            # :49-51
                 tmp = _int_matmul(p8, vj)                                    # :59 int32 accumulator
+                if vs_blocked:                                               # csrc/mask.h:335
+                    vs = v_scale.float()[:, :, start_n // v_scale_block][:, :, None, :]
                 tmp = tmp * vs / 127                                         # :61
                 a = a + tmp                                                  # :62
             else:
@@ -214,10 +249,12 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
 
 def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float, *,
                         block_m: int = 128, block_n: int = 128, out_dtype=torch.float16,
-                        p_requant=p_requant_reference, return_lse: bool = False):
-    """Full-int8 forward, flash_atten_full_int8.py (see module docstring for line map)."""
+                        p_requant=p_requant_reference, return_lse: bool = False,
+                        v_scale_block: Optional[int] = None):
+    """Full-int8 forward, flash_atten_full_int8.py (see module docstring for line map).  ``v_scale`` is [B,H] (the
+    reference's Python API) or [B,H,ceil(N/v_scale_block),d] (the layout of its CUDA kernel)."""
     acc, l, m = _blocked_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale,
-                                 block_m, block_n, p_requant=p_requant)
+                                 block_m, block_n, p_requant=p_requant, v_scale_block=v_scale_block)
     o = (acc / l[..., None]).to(out_dtype)                                   # :181-182
     if return_lse:
         return o, m + torch.log2(l)
@@ -283,7 +320,8 @@ def splitkv_ranges_causal(n_keys: int, block_m: int, block_n: int, num_splits: i
 
 
 def attention_full_int8_splitkv(q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float, num_splits: int, *,
-                                block_m: int = 128, block_n: int = 128, out_dtype=torch.float16):
+                                block_m: int = 128, block_n: int = 128, out_dtype=torch.float16,
+                                v_scale_block: Optional[int] = None):
     """Full-int8 forward evaluated as ``num_splits`` independent key ranges merged by ``splitkv_combine``: the ranges of
     ``splitkv_ranges`` for a non-causal pass, those of ``splitkv_ranges_causal`` (per row tile) for a causal one."""
     B, H, N, D = q.shape
@@ -299,7 +337,7 @@ def attention_full_int8_splitkv(q, k, v, q_scale, k_scale, v_scale, causal: bool
             continue
         acc, l, m = _blocked_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale,
                                      block_m, block_n, key_lo=b0 * block_n, key_hi=min(b1 * block_n, N),
-                                     row_lo=r0, row_hi=r1)
+                                     row_lo=r0, row_hi=r1, v_scale_block=v_scale_block)
         seen = ~torch.isinf(m[:, :, r0:r1])          # rows above the split's range saw no key
         a, ll, mm = acc[:, :, r0:r1], l[:, :, r0:r1], m[:, :, r0:r1]
         o_parts[s, :, :, r0:r1] = torch.where(seen[..., None], a / ll[..., None], torch.zeros_like(a))

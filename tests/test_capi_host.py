@@ -80,6 +80,10 @@ def _valid_block():
     (lambda p: setattr(p, "q_stride_n", 64), -7),          # rows overlap: stride below head_dim
     (lambda p: (setattr(p, "seqlen", 1 << 20), setattr(p, "k_stride_n", 1 << 13)), -7),   # a K slice of 8 GiB
     (lambda p: (setattr(p, "num_splits", 65), setattr(p, "workspace", 0x10000), setattr(p, "workspace_bytes", 1 << 40)), -8),
+    (lambda p: (setattr(p, "v_scale_block", 64), setattr(p, "vs_stride_blk", 128)), -9),    # not a multiple of the key block (128)
+    (lambda p: (setattr(p, "v_scale_block", 128), setattr(p, "vs_stride_blk", 64)), -9),    # scale rows overlap
+    (lambda p: setattr(p, "v_scale_block", -1), -9),
+    (lambda p: (setattr(p, "v_scale_block", 128), setattr(p, "vs_stride_blk", 128), setattr(p, "v_scale", 0x10002)), -4),
 ])
 def test_validation_rejects_bad_blocks_before_touching_the_gpu(mutate, code):
     lib = _capi.load()

@@ -325,3 +325,82 @@ def test_exact_attention_matches_reference_recipe():
     got = O.attention_exact(q, k, v, True, 1.0).float()
     want = _dense_attention(q.float() @ k.float().transpose(2, 3), v.float(), True)
     assert (got - want).abs().max() < 2e-3
+
+
+# ---- per-block, per-channel V scales (layout of the reference's CUDA kernel, csrc/flash_fwd_kernel_full_qi8.h:156-160)
+def test_quant_perblock_channel_against_python_loop_and_invariants():
+    g = torch.Generator().manual_seed(12)
+    x = (torch.randn((1, 2, 20, 4), generator=g) * 2).half()
+    x[0, 1, 8:16, 2] = 0                                       # an all-zero (block, channel)
+    q, s = O.quant_perblock_channel(x, 8)
+    assert q.dtype == torch.int8 and q.shape == x.shape and s.shape == (1, 2, 3, 4) and s.dtype == torch.float32
+    for h in range(2):
+        for blk in range(3):
+            rows = range(8 * blk, min(8 * blk + 8, 20))
+            for c in range(4):
+                col = [np.float32(float(x[0, h, r, c])) for r in rows]
+                amax = max(abs(t) for t in col)
+                sc = np.float32(amax) / np.float32(127)
+                assert float(s[0, h, blk, c]) == float(sc)
+                for r, t in zip(rows, col):
+                    want = 0 if sc == 0 else int(np.rint(np.float32(t) / sc))
+                    assert int(q[0, h, r, c]) == want
+                if amax > 0:
+                    assert max(abs(int(q[0, h, r, c])) for r in rows) == 127
+    assert int(q[0, 1, 8:16, 2].abs().max()) == 0 and float(s[0, 1, 1, 2]) == 0.0
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_blocked_v_scale_filled_with_the_scalar_is_the_scalar_form(causal):
+    q, k, v, _ = O.make_inputs(1, 2, 192, 32, seed=13)
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    want = O.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, 0.2, block_m=64, block_n=64)
+    vs4 = vs.float()[:, :, None, None].expand(1, 2, 3, 32).contiguous()
+    got = O.attention_full_int8(q8, k8, v8, qs, ks, vs4, causal, 0.2, block_m=64, block_n=64, v_scale_block=64)
+    assert torch.equal(got, want)
+    vs4b = vs.float()[:, :, None, None].expand(1, 2, 2, 32).contiguous()         # one scale row per two key blocks
+    got = O.attention_full_int8(q8, k8, v8, qs, ks, vs4b, causal, 0.2, block_m=64, block_n=64, v_scale_block=128)
+    assert torch.equal(got, want)
+
+
+def test_blocked_v_scale_equals_scalar_form_on_prescaled_v():
+    # power-of-two factors per (block, channel) commute exactly with the integer products: scaling V8 by 2^e and
+    # using the scalar form gives the same fp32 numbers as the factors applied to the accumulator, as long as the
+    # scaled V stays exactly representable (done here in the integer domain with small V)
+    g = torch.Generator().manual_seed(14)
+    q, k, _, _ = O.make_inputs(1, 1, 128, 16, seed=14)
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k)
+    v8 = torch.randint(-15, 16, (1, 1, 128, 16), generator=g, dtype=torch.int8)
+    e = torch.randint(0, 4, (1, 1, 2, 16), generator=g)
+    fac = torch.pow(2.0, e.float())                                              # [1,1,2,16], block of 64 keys
+    v8_scaled = (v8.view(1, 1, 2, 64, 16).float() * fac[:, :, :, None, :]).view(1, 1, 128, 16).to(torch.int8)
+    assert int(v8_scaled.abs().max()) <= 127
+    one = torch.ones((1, 1))
+    want = O.attention_full_int8(q8, k8, v8_scaled, qs, ks, one, False, 0.3, block_m=64, block_n=64, out_dtype=torch.float32)
+    got = O.attention_full_int8(q8, k8, v8, qs, ks, fac, False, 0.3, block_m=64, block_n=64, v_scale_block=64,
+                                out_dtype=torch.float32)
+    assert torch.equal(got, want)
+
+
+def test_blocked_v_scale_is_more_accurate_with_an_outlier_channel_burst():
+    q, k, v, _ = O.make_inputs(1, 2, 256, 32, seed=15)
+    v = v.clone(); v[:, :, 64:128, 5] *= 30                                     # a burst in one channel of one key block
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k)
+    exact = O.attention_exact(q, k, v, False, 0.2).float()
+    v8s, vss = O.quant_pertensor(v)
+    coarse = O.attention_full_int8(q8, k8, v8s, qs, ks, vss, False, 0.2, block_m=64, block_n=64).float()
+    v8b, vsb = O.quant_perblock_channel(v, 64)
+    fine = O.attention_full_int8(q8, k8, v8b, qs, ks, vsb, False, 0.2, block_m=64, block_n=64, v_scale_block=64).float()
+    other = [c for c in range(32) if c != 5]
+    err_c = (coarse - exact)[..., other].abs().mean()
+    err_f = (fine - exact)[..., other].abs().mean()
+    assert err_f < 0.5 * err_c                                                   # the burst no longer sets every channel's step
+
+
+def test_blocked_v_scale_split_agrees_with_single_pass():
+    q, k, v, _ = O.make_inputs(1, 2, 256, 32, seed=16)
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_perblock_channel(v, 64)
+    one = O.attention_full_int8(q8, k8, v8, qs, ks, vs, False, 0.2, block_m=64, block_n=64, v_scale_block=64).float()
+    two = O.attention_full_int8_splitkv(q8, k8, v8, qs, ks, vs, False, 0.2, 2, block_m=64, block_n=64, v_scale_block=64).float()
+    # (the second split quantises P against its own maximum: same size of deviation as with a scalar V scale)
+    assert (one - two).abs().max() < 3e-2 and (one - two).abs().mean() < 2e-3
