@@ -3,6 +3,7 @@
 #include "intfa_device.h"
 #include "intfa_launch.h"
 #include "intfa_splitkv.h"
+#include "intfa_fwd_decode.h"
 
 using namespace intfa;
 
@@ -118,6 +119,13 @@ int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t str
     return e == hipSuccess ? INTFA_OK : (int)e;
 }
 
+// Few query rows per head and no causal mask (decoding against a cache): the full-int8 pass runs the kernel whose waves
+// share the keys of a block instead of each taking 32 query rows.
+constexpr int kDecodeMaxRows = 2 * kDecodeRows;
+bool decode_shaped(int variant, int seqlen, int causal) {
+    return variant == INTFA_VARIANT_FULL_INT8 && !causal && seqlen <= kDecodeMaxRows;
+}
+
 int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dump_s, hipStream_t stream) {
     const bool vblk = variant == INTFA_VARIANT_FULL_INT8 && !dump_s && kp.vs_g > 0;
     LaunchSel sel;
@@ -127,7 +135,11 @@ int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dum
     sel.split = kp.num_splits > 1;
     sel.dump_s = dump_s;
     const int d = kp.head_dim;
-    if (vblk) {
+    if (!dump_s && decode_shaped(variant, kp.seqlen, kp.causal)) {
+        if (d == 64) return launch_decode_full_int8_d64(kp, sel, stream);
+        if (d == 128) return launch_decode_full_int8_d128(kp, sel, stream);
+        if (d == 256) return launch_decode_full_int8_d256(kp, sel, stream);
+    } else if (vblk) {
         if (d == 64) return launch_full_int8_vblk_d64(kp, sel, stream);
         if (d == 128) return launch_full_int8_vblk_d128(kp, sel, stream);
         if (d == 256) return launch_full_int8_vblk_d256(kp, sel, stream);
@@ -199,7 +211,8 @@ int intfa_fwd_suggest_splits(const intfa_fwd_params* p, int variant, int num_cus
     const int cus = num_cus > 0 ? num_cus : 256;
     const int64_t slots = 2ll * cus;                                           // two workgroups per compute unit
     int64_t wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kBlockM - 1) / kBlockM);
-    if (variant == INTFA_VARIANT_FULL_INT8 && p->head_dim == 256) wgs *= 2;     // column halves
+    if (decode_shaped(variant, p->seqlen, p->causal)) wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kDecodeRows - 1) / kDecodeRows);
+    else if (variant == INTFA_VARIANT_FULL_INT8 && p->head_dim == 256) wgs *= 2;     // column halves
     if (wgs * 5 >= slots * 4) return 1;                                        // at least 80 % of the slots are used anyway
     const int seqlen_k = p->seqlen_k > 0 ? p->seqlen_k : p->seqlen;
     const int bn = block_n_for(variant, p->head_dim);

@@ -32,6 +32,8 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef short v4s __attribute__((ext_vector_type(4)));
 
 #define INTFA_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+// compile-time switch passed as a lambda argument (selects the LDS buffer or the masked code instance of a pipeline step)
+template <bool V> struct BoolTag { static constexpr bool value = V; };
 #define INTFA_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
 
 constexpr int kBlockM = 128;

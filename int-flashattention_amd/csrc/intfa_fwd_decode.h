@@ -1,0 +1,348 @@
+// Full-int8 forward for few query rows per head (decoding against a key/value cache, Nq << Nk).
+//
+// Same arithmetic as fwd_full_int8_kernel (flash_atten_full_int8.py:9-71 per 128-key block: int32 S, dequantise, running
+// max, P = exp2(X c - m), P requantised with the fixed scale 127, int32 P V, fp32 accumulator), other division of labour.
+// The general kernel gives each of its four waves 32 query rows; with one or a few query rows three of them would redo
+// the first one's work on padding while the pass is bound by streaming K and V from HBM.  Here one workgroup owns 32
+// query rows and its four waves share every key block:
+//   * wave w computes S^T for keys 32w .. 32w+31 of the block (KS MFMAs), dequantises and takes the partial row maxima;
+//   * the partial maxima meet in LDS (barrier), every wave then holds the block's row maximum;
+//   * wave w exponentiates and requantises its 32 keys and publishes its P8 fragment in LDS (barrier);
+//   * wave w multiplies the whole block's P (all four fragments) with ITS 32-column slice of V and updates its slice of
+//     the fp32 output; the partial row sums of P meet once, in the epilogue.
+// The int32 sums run over the same 128 keys as in the general kernel, so results agree with it up to the order of the
+// fp32 additions of the row sums.  K/V tiles are double-buffered in LDS and the whole next tile is requested at the
+// start of a block (the data comes from HBM, not from a cache shared with other query blocks).
+#pragma once
+#include "intfa_device.h"
+
+namespace intfa {
+
+constexpr int kDecodeRows = 32;       // query rows per workgroup of the decode kernel
+
+template <int D, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool SPLIT, bool VBLK>
+__global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const KParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
+    constexpr int KS = D / 32;                   // k-steps of Q K^T
+    constexpr int DT = D / 32;                   // 32-wide output tiles along head_dim; wave w owns tiles w, w+4, ...
+    constexpr int DTW = (DT + 3) / 4;            // output tiles per wave
+    constexpr int NST = 4, BN = 32 * NST;        // one 32-key sub-tile per wave
+    constexpr int KT = BN * D, VT = BN * D;      // bytes of one K / V tile
+    constexpr int CH = D / 16;                   // 16-byte chunks per row
+    constexpr int SWM = (CH < 8 ? CH : 8) - 1;   // swizzle mask of V rows
+    // LDS map (bytes)
+    constexpr int OFF_KS = 0;                            // two fp32 k_scale vectors
+    constexpr int OFF_XM = 2 * BN * 4;                   // 4 waves x 32 rows fp32: partial row maxima / row sums
+    constexpr int OFF_XP = OFF_XM + 4 * 32 * 4;          // 4 waves x 64 lanes x 16 bytes: the waves' P8 fragments
+    constexpr int OFF_VS = OFF_XP + 4 * 64 * 16;         // VBLK: two vectors of D fp32 channel scales
+    constexpr int OFF_K = OFF_VS + (VBLK ? 2 * D * 4 : 0);
+    constexpr int OFF_V = OFF_K + 2 * KT;
+    constexpr int LDS_BYTES = OFF_V + 2 * VT;
+    static_assert(OFF_K % 256 == 0, "tiles keep the bank alignment the swizzles assume");
+    __shared__ __attribute__((aligned(1024))) char smem[LDS_BYTES];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lq = lane & 31, lh = lane >> 5;
+
+    // ---- block -> (head, 32-row query block, split); whole K/V heads go to one XCD as in the general kernel
+    const int n_mblk = (p.seqlen + kDecodeRows - 1) / kDecodeRows;
+    const int n_split = SPLIT ? p.num_splits : 1;
+    const int per_head = n_mblk * n_split;
+    const int n_heads = p.batch * p.heads;
+    const int bid = blockIdx.x;
+    const int kv_group = p.kv_group;
+    const int per_kv = per_head * kv_group;
+    const int n_kv = n_heads / kv_group;
+    int head, rem;
+    {
+        int kv_lin, r;
+        if ((n_kv & 7) == 0) {
+            const int xcd = bid & 7, slot = bid >> 3;
+            kv_lin = (slot / per_kv) * 8 + xcd;
+            r = slot % per_kv;
+        } else {
+            kv_lin = bid / per_kv;
+            r = bid % per_kv;
+        }
+        const int heads_kv = p.heads / kv_group;
+        const int bb = kv_lin / heads_kv, hk_ = kv_lin % heads_kv;
+        head = bb * p.heads + hk_ * kv_group + r / per_head;
+        rem = r % per_head;
+    }
+    const int mb = rem / n_split, split = rem % n_split;
+    const int b = head / p.heads, h = head % p.heads;
+    const int hk = h / kv_group;
+
+    const int nb_total = (p.seqlen_k + BN - 1) / BN;
+    int nb_begin = 0, nb_end = nb_total;
+    if (SPLIT) {                                           // csrc/flash_fwd_kernel.h:503-511
+        nb_begin = split * p.blocks_per_split;
+        const int e = nb_begin + p.blocks_per_split;
+        nb_end = e < nb_end ? e : nb_end;
+    }
+    const int q_row = mb * kDecodeRows + lq;
+    const bool q_valid = q_row < p.seqlen;
+    const int q_ld = q_valid ? q_row : p.seqlen - 1;
+
+    // ---- Q fragment (B operand of S^T = K Q^T), the same 32 rows in every wave
+    v4i qreg[KS];
+    {
+        const char* qrow = p.q + b * p.q_sb + h * p.q_sh + (int64_t)q_ld * p.q_sn;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qreg[ks] = *(const v4i*)(qrow + ks * 32 + lh * 16);
+    }
+    const float qs = load_scale(p.q_scale, b * p.qs_sb + h * p.qs_sh + (int64_t)q_ld * p.qs_sn, p.scale_dtype);
+    const float qsc = qs * p.qk_scale_log2;
+
+    float m_run = -INFINITY, l_run = 0.f;        // l_run: this wave's keys only
+    float o_acc[DTW][16];
+#pragma unroll
+    for (int j = 0; j < DTW; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[j][r] = 0.f;
+
+    // ---- global -> LDS copies (asynchronous, straight into LDS; the four waves split the instructions)
+    const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
+    const char* Vg = p.v + b * p.v_sb + hk * p.v_sh;
+    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen_k - 1) * p.k_sn + D));
+    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen_k - 1) * p.v_sn + D));
+    const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
+    const auto k_lane = tile_load_lane<D, SWZ_K, BN>(k_sn, wave, lane);
+    const auto v_lane = tile_load_lane<D, SWZ_V8, BN>(v_sn, wave, lane);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    auto issue_loads = [&](int nb, int buf) __attribute__((always_inline)) {
+        issue_tile_load<D, SWZ_K, BN>(k_rsrc, (uint32_t)(nb * BN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane);
+        issue_tile_load<D, SWZ_V8, BN>(v_rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane);
+    };
+    // k_scale of a block: thread t < 128 fetches the scale of key t; converted to fp32 when stored to LDS
+    const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
+    const char* Ksg = p.k_scale + (b * p.ks_sb + hk * p.ks_sh) * ks_esize;
+    const int ks_stride = (int)(p.ks_sn * ks_esize);
+    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
+        int key = nb * BN + (tid & (BN - 1));
+        key = key < p.seqlen_k ? key : p.seqlen_k - 1;                  // keys past the end are masked later
+        const char* src = Ksg + (int64_t)key * ks_stride;
+        if (p.scale_dtype == 2) return *(const uint32_t*)src;
+        return (uint32_t)*(const uint16_t*)src;
+    };
+    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float {
+        if (p.scale_dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+        if (p.scale_dtype == 1) return __builtin_bit_cast(float, raw << 16);
+        return __builtin_bit_cast(float, raw);
+    };
+    // VBLK: fp32 channel scales of a key block; thread 128 + c fetches channel c (D = 256: threads 0 .. 255)
+    const int vs_c = D <= 128 ? tid - 128 : tid;
+    const bool vs_thread = VBLK && vs_c >= 0 && vs_c < D;
+    const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + (vs_thread ? vs_c : 0));
+    auto load_vs = [&](int nb) __attribute__((always_inline)) -> float {
+        if (!VBLK) return 0.f;
+        const int row = p.vs_g == 1 ? nb : nb / p.vs_g;
+        return Vsg[(int64_t)row * p.vs_sblk];
+    };
+
+    // ---- per-lane LDS offsets
+    const int k_swz = swz_k<D>(lq) & (CH - 1);
+    uint32_t k_rd[KS];                            // this wave's 32 keys: row 32*wave + lq, chunk 2*ks + lh
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) k_rd[ks] = OFF_K + (32 * wave + lq) * D + (((2 * ks + lh) ^ k_swz) << 4);
+    // V through the transposing 8-byte load (see fwd_full_int8_kernel): source lane s of a 16-lane group points at key
+    // row 8*(j>>2) + 4*lh + (j&3), j = s/2 (+16 for the second load, +32 per sub-tile), 8-byte half s&1
+    const int g16 = lane >> 4, i16 = lane & 15, jj = i16 >> 1;
+    const int v_row0 = 8 * (jj >> 2) + 4 * lh + (jj & 3);
+    const int v_swz = swz_v8<D>(v_row0) & SWM;
+    uint32_t v_rd[DTW];
+#pragma unroll
+    for (int j = 0; j < DTW; ++j) {
+        const int dt = wave + 4 * j;
+        const int c = 2 * dt + (g16 & 1);
+        v_rd[j] = OFF_V + v_row0 * D + 8 * (i16 & 1) + (((c & SWM) ^ v_swz) << 4) + ((c & ~SWM) << 4);
+    }
+    const uint32_t ks_rd = OFF_KS + 4 * (32 * wave) + 16 * lh;       // + 4 * 8*a4 per read
+    const uint32_t ks_wr = OFF_KS + 4 * (tid & (BN - 1));
+    const uint32_t xm_wr = OFF_XM + 4 * (32 * wave + lq);
+    const uint32_t xm_rd = OFF_XM + 4 * lq;                          // + 128 per wave
+    const uint32_t xp_wr = OFF_XP + 1024 * wave + 16 * lane;
+    const uint32_t xp_rd = OFF_XP + 16 * lane;                       // + 1024 per wave
+    const uint32_t vs_wr = OFF_VS + 4 * (vs_thread ? vs_c : 0);
+    const uint32_t vs_rd = OFF_VS + 16 * lh;                         // + 4 * (32*dt + 8*a4) per read
+    const bool own_tile0 = wave < DT;                                // head_dim 64: waves 2 and 3 own no output tile
+    const int tail_keys = p.seqlen_k - (nb_total - 1) * BN;          // valid keys of the last block
+
+    auto step = [&](auto buf_tag, int nb) __attribute__((always_inline)) {
+        constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
+        constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4, VSB = BUF * D * 4;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();                                   // tile nb has landed; the other buffer and the exchange areas are free
+        const bool more = nb + 1 < nb_end;
+        uint32_t ks_next = 0;
+        float vs_next = 0.f;
+        if (more) {
+            issue_loads(nb + 1, BUF ^ 1);
+            if (tid < BN) ks_next = load_ks(nb + 1);
+            if (vs_thread) vs_next = load_vs(nb + 1);
+        }
+        // -------- S^T of this wave's 32 keys, dequantise, partial row maximum
+        v4i fr[KS];
+        v4f kk[4];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) fr[ks] = *(const v4i*)(smem + k_rd[ks] + KB);
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) kk[a4] = *(const v4f*)(smem + ks_rd + SB + 4 * 8 * a4);
+        v16i sacc = (v16i){0};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) sacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[ks], qreg[ks], sacc, 0, 0, 0);
+        // V fragments of this wave's output tiles travel during the softmax
+        v4i vf[DTW][NST];
+#pragma unroll
+        for (int j = 0; j < DTW; ++j)
+#pragma unroll
+            for (int st = 0; st < NST; ++st) {
+                const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                    (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[j] + VB + (32 * st) * D));
+                const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                    (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[j] + VB + (32 * st + 16) * D));
+                vf[j][st] = (v4i){lo[0], lo[1], hi[0], hi[1]};
+            }
+        float x[16];
+        float mx = -INFINITY;
+        const bool tail = nb == nb_total - 1 && tail_keys < BN;          // wave-uniform
+        const int key_lim = tail_keys - 32 * wave - 4 * lh;              // keys of this lane with 8*a4 + b4 >= key_lim are past the end
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float v = (float)sacc[r] * kk[r >> 2][r & 3];
+            if (tail && 8 * (r >> 2) + (r & 3) >= key_lim) v = -INFINITY;
+            x[r] = v;
+            mx = fmaxf(mx, v);
+        }
+        mx = half_pair_max(mx);
+        if (lh == 0) *(float*)(smem + xm_wr) = mx;
+        __syncthreads();                                   // the four partial maxima are in LDS
+        mx = fmaxf(fmaxf(*(const float*)(smem + xm_rd), *(const float*)(smem + xm_rd + 128)),
+                   fmaxf(*(const float*)(smem + xm_rd + 256), *(const float*)(smem + xm_rd + 384)));
+        const float m_new = fmaxf(m_run, mx * qsc);
+        const float alpha = fast_exp2(m_run - m_new);
+        m_run = m_new;
+        // -------- P of this wave's keys, requantised; partial row sum
+        const float bias = (PROUND == 0 ? kLog2_127 : 0.f) - m_new;
+        float lsum = 0.f;
+        v4i p8;
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4) {
+            unsigned pk = 0;
+#pragma unroll
+            for (int b4 = 0; b4 < 4; ++b4) {
+                const float e = fast_exp2(fmaf(x[4 * w4 + b4], qsc, bias));      // RNE mode: 127 * p
+                lsum += e;
+                if (PROUND == 0) {
+                    pk = __builtin_amdgcn_cvt_pk_u8_f32(e, b4, pk);
+                } else {
+                    // the reference's fp16 chain: fp16(p) * 127 -> fp16, + 0.5 -> fp16, truncate (flash_atten_full_int8.py:49-51)
+                    _Float16 hp = (_Float16)e;
+                    hp = hp * (_Float16)127.0f;
+                    hp = hp + (_Float16)0.5f;
+                    pk |= (unsigned)(int)hp << (8 * b4);
+                }
+            }
+            p8[w4] = (int)pk;
+        }
+        *(v4i*)(smem + xp_wr) = p8;
+        v4f vsc[DTW][4];
+        if (VBLK) {
+#pragma unroll
+            for (int j = 0; j < DTW; ++j)
+#pragma unroll
+                for (int a4 = 0; a4 < 4; ++a4) vsc[j][a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (32 * (wave + 4 * j) + 8 * a4));
+        }
+        __syncthreads();                                   // the four P8 fragments are in LDS
+        v4i pall[NST];
+#pragma unroll
+        for (int st = 0; st < NST; ++st) pall[st] = *(const v4i*)(smem + xp_rd + 1024 * st);
+        // -------- this wave's output columns: O^T[d, q] += V^T[d, key] P^T[key, q] over the whole block
+#pragma unroll
+        for (int j = 0; j < DTW; ++j) {
+            if (j == 0 ? !own_tile0 : false) continue;
+            v16i acc = (v16i){0};
+#pragma unroll
+            for (int st = 0; st < NST; ++st) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[j][st], pall[st], acc, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                if (VBLK) o_acc[j][r] = fmaf(o_acc[j][r], alpha, (float)acc[r] * vsc[j][r >> 2][r & 3]);
+                else o_acc[j][r] = fmaf(o_acc[j][r], alpha, (float)acc[r]);
+            }
+        }
+        l_run = fmaf(l_run, alpha, lsum);
+        if (more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
+        if (more && vs_thread) *(float*)(smem + vs_wr + (BUF ^ 1) * D * 4) = vs_next;
+    };
+
+    if (nb_begin < nb_end) {
+        issue_loads(nb_begin, 0);
+        if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(load_ks(nb_begin));
+        if (vs_thread) *(float*)(smem + vs_wr) = load_vs(nb_begin);
+        int nb = nb_begin;
+        while (true) {
+            if (nb >= nb_end) break;
+            step(BoolTag<false>{}, nb++);
+            if (nb >= nb_end) break;
+            step(BoolTag<true>{}, nb++);
+        }
+    }
+
+    // ---- epilogue: the waves' partial row sums meet in LDS; every wave scales and stores its own output columns
+    __syncthreads();
+    const float l_pair = half_pair_sum(l_run);
+    if (lh == 0) *(float*)(smem + xm_wr) = l_pair;
+    __syncthreads();
+    const float l_tot = (*(const float*)(smem + xm_rd) + *(const float*)(smem + xm_rd + 128)) +
+                        (*(const float*)(smem + xm_rd + 256) + *(const float*)(smem + xm_rd + 384));   // units of 1/127 when PROUND == 0
+    const float vs = VBLK ? 1.f : load_scale(p.v_scale, b * p.vs_sb + hk * p.vs_sh, p.scale_dtype);
+    const float out_scale = (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
+    const float l_true = (PROUND == 0) ? l_tot * (1.f / 127.f) : l_tot;
+    const float lse = m_run + __builtin_log2f(l_true);
+    const bool seen = nb_begin < nb_end;
+    if (!q_valid) return;
+    if (SPLIT) {
+        const int64_t row = ((int64_t)(split * p.batch + b) * p.heads + h) * p.seqlen + q_row;
+        float* op = p.o_part + row * D;
+#pragma unroll
+        for (int j = 0; j < DTW; ++j) {
+            const int dt = wave + 4 * j;
+            if (dt >= DT) continue;
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4) {
+                v4f o;
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[j][4 * a4 + b4] * out_scale : 0.f;
+                *(v4f*)(op + 32 * dt + 8 * a4 + 4 * lh) = o;
+            }
+        }
+        if (wave == 0 && lh == 0) p.lse_part[row] = seen ? lse : -INFINITY;
+        return;
+    }
+    char* orow = p.out + b * p.o_sb + h * p.o_sh + (int64_t)q_row * p.o_sn;
+#pragma unroll
+    for (int j = 0; j < DTW; ++j) {
+        const int dt = wave + 4 * j;
+        if (dt >= DT) continue;
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+            const int d0 = 32 * dt + 8 * a4 + 4 * lh;
+            if (OUT_DT == 0) {
+                v4h o;
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(o_acc[j][4 * a4 + b4] * out_scale);
+                *(v4h*)(orow + d0 * 2) = o;
+            } else {
+                v4s o;
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(o_acc[j][4 * a4 + b4] * out_scale);
+                *(v4s*)(orow + d0 * 2) = o;
+            }
+        }
+    }
+    if (p.lse != nullptr && wave == 0 && lh == 0) p.lse[((int64_t)b * p.heads + h) * p.seqlen + q_row] = lse;
+#endif  // __HIP_DEVICE_COMPILE__
+}
+
+}  // namespace intfa

@@ -16,8 +16,6 @@
 
 namespace intfa {
 
-template <bool V> struct BoolTag { static constexpr bool value = V; };
-
 // Key block length of the full-int8 kernel: 128 keys, or 64 at head_dim 256 (registers and LDS).
 template <int D> struct FullInt8Geom {
     static constexpr int NST = D <= 128 ? 4 : 2;

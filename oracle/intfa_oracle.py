@@ -41,6 +41,8 @@ How every function is pinned (tests/test_oracle.py):
   is that constant times sum(P8)/(127 l).
 * causal: equality with a dense tril-masked evaluation; first row attends to key 0 only.
 * split-KV: any split count agrees with one split to fp32 rounding.
+* separate query and key lengths (non-causal): rows are independent, so a slice of the query rows against the full keys
+  must reproduce the same rows of the square evaluation bit for bit.
 * blocked V scales: a 4-D scale tensor filled with one value per (batch, head) reproduces the scalar form bit for
   bit; the result equals the scalar form applied to V pre-multiplied by the block/channel factors when these are
   powers of two; ``quant_perblock_channel`` against a pure-Python loop, and every (block, channel) reaches +-127.
@@ -176,13 +178,15 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
     (csrc/mask.h:313-340); ``v_scale_block`` must be a multiple of ``block_n``.
     """
     B, H, N, D = q.shape
-    key_hi = N if key_hi is None else key_hi
+    Nk = k.shape[2]                # differs from N for cross attention / decoding against a cache (non-causal only)
+    assert not causal or Nk == N   # the reference's mask is defined for one N_CTX (flash_atten_full_int8.py:213)
+    key_hi = Nk if key_hi is None else key_hi
     row_hi = N if row_hi is None else row_hi
     # N need not be a multiple of the blocks: the last key block and the last row tile are simply shorter, which is
     # what masking the missing keys with -inf amounts to (csrc/mask.h:261-263 for the reference's CUDA tree; its Triton
     # kernels have no bounds handling at all)
     assert block_m % block_n == 0
-    assert key_lo % block_n == 0 and (key_hi % block_n == 0 or key_hi == N)
+    assert key_lo % block_n == 0 and (key_hi % block_n == 0 or key_hi == Nk)
     qk_scale = float(torch.tensor(sm_scale, dtype=torch.float32) * torch.tensor(LOG2E, dtype=torch.float32))
     m = torch.full((B, H, N), float("-inf"), dtype=torch.float32)
     l = torch.ones((B, H, N), dtype=torch.float32)          # flash_atten_full_int8.py:153
@@ -194,7 +198,7 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
     vs_blocked = variant == "full" and v_scale.dim() == 4
     if vs_blocked:
         v_scale_block = block_n if v_scale_block is None else v_scale_block
-        assert v_scale_block % block_n == 0 and v_scale.shape[2] == (k.shape[2] + v_scale_block - 1) // v_scale_block
+        assert v_scale_block % block_n == 0 and v_scale.shape[2] == (Nk + v_scale_block - 1) // v_scale_block
     elif variant == "full":
         vs = v_scale.float()[:, :, None, None]
     rows = torch.arange(N)
@@ -331,12 +335,12 @@ def attention_full_int8_splitkv(q, k, v, q_scale, k_scale, v_scale, causal: bool
         jobs = [(s, r0, r1, b0, b1) for r0, r1, ranges in splitkv_ranges_causal(N, block_m, block_n, num_splits)
                 for s, (b0, b1) in enumerate(ranges)]
     else:
-        jobs = [(s, 0, N, b0, b1) for s, (b0, b1) in enumerate(splitkv_ranges(N, block_n, num_splits))]
+        jobs = [(s, 0, N, b0, b1) for s, (b0, b1) in enumerate(splitkv_ranges(k.shape[2], block_n, num_splits))]
     for s, r0, r1, b0, b1 in jobs:
         if b0 >= b1:
             continue
         acc, l, m = _blocked_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale,
-                                     block_m, block_n, key_lo=b0 * block_n, key_hi=min(b1 * block_n, N),
+                                     block_m, block_n, key_lo=b0 * block_n, key_hi=min(b1 * block_n, k.shape[2]),
                                      row_lo=r0, row_hi=r1, v_scale_block=v_scale_block)
         seen = ~torch.isinf(m[:, :, r0:r1])          # rows above the split's range saw no key
         a, ll, mm = acc[:, :, r0:r1], l[:, :, r0:r1], m[:, :, r0:r1]

@@ -1,0 +1,124 @@
+"""GPU parity of the decode-shaped full-int8 forward (few query rows per head against a long key/value cache): the
+kernel whose four waves share each key block, through the C ABI, against the CPU oracle evaluated with separate query
+and key lengths at the kernel's key-block length."""
+import pytest
+import torch
+
+import intfa_oracle as O
+import int_flashattention_amd as M
+from test_gpu_parity import DEV, MAX_ABS, MEAN_REL, assert_same_rounding, gpu, max_abs, mean_rel
+
+pytestmark = pytest.mark.gpu
+
+
+def decode_inputs(B, H, H_kv, Nq, Nk, D, seed, dtype=torch.float16, v_block=None):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((B, H, Nq, D), generator=g).to(dtype)
+    k = torch.randn((B, H_kv, Nk, D), generator=g).to(dtype)
+    v = torch.randn((B, H_kv, Nk, D), generator=g).to(dtype)
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k)
+    v8, vs = O.quant_perblock_channel(v, v_block) if v_block else O.quant_pertensor(v)
+    return dict(q=q, k=k, v=v, q8=q8, k8=k8, v8=v8, qs=qs, ks=ks, vs=vs, g=H // H_kv)
+
+
+def oracle(x, sm, bn, **kw):
+    rep = lambda t: t.repeat_interleave(x["g"], dim=1)
+    return O.attention_full_int8(x["q8"], rep(x["k8"]), rep(x["v8"]), x["qs"], rep(x["ks"]), rep(x["vs"]), False, sm,
+                                 block_n=bn, **kw)
+
+
+@pytest.mark.parametrize("B,H,H_kv,Nq,Nk,D", [
+    (2, 4, 4, 1, 1000, 128),        # one query per head, ragged cache length
+    (1, 8, 2, 1, 2048, 128),        # grouped heads: the wrapper folds a group's 4 heads into 4 rows of one head
+    (2, 2, 2, 5, 777, 64),          # head_dim 64: two of the four waves own an output tile
+    (1, 2, 2, 32, 640, 128),        # a full 32-row tile
+    (1, 2, 2, 33, 513, 128),        # two 32-row workgroups per head, the second with one valid row
+    (1, 3, 3, 64, 130, 256),        # head_dim 256: two output tiles per wave
+    (1, 2, 1, 7, 96, 128),          # cache shorter than one key block
+    (1, 2, 2, 2, 1, 64),            # a single key
+])
+@pytest.mark.parametrize("p_round", ["rne", "reference"])
+def test_decode_matches_oracle(B, H, H_kv, Nq, Nk, D, p_round):
+    x = decode_inputs(B, H, H_kv, Nq, Nk, D, seed=90)
+    sm = D ** -0.5
+    bn = M.block_n("full", 128)       # the decode kernel takes 128 keys per block at every head_dim
+    o, lse = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, sm, p_round=p_round,
+                                   return_lse=True)
+    torch.cuda.synchronize()
+    assert o.shape == (B, H, Nq, D) and o.dtype == torch.float16 and torch.isfinite(o).all()
+    ref, lse_ref = oracle(x, sm, bn, return_lse=True)
+    assert max_abs(o, ref) <= MAX_ABS and mean_rel(o, ref) <= MEAN_REL
+    same = ref if p_round == "reference" else oracle(x, sm, bn, p_requant=O.p_requant_rne)
+    if Nk >= 64:
+        assert_same_rounding(o, same)
+    else:                                 # a handful of keys: one P8 step is a large share of a row
+        assert max_abs(o, same) <= MAX_ABS
+    assert (lse.cpu() - lse_ref).abs().max().item() < 1e-3
+
+
+@pytest.mark.parametrize("splits", [2, 5, "auto"])
+def test_decode_split_kv_matches_oracle_split(splits):
+    x = decode_inputs(2, 4, 4, 3, 2000, 128, seed=91)
+    sm = 128 ** -0.5
+    args = gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"])
+    o = M.attention_full_int8(*args, False, sm, num_splits=splits, p_round="reference")
+    torch.cuda.synchronize()
+    single = oracle(x, sm, 128)
+    assert max_abs(o, single) <= MAX_ABS and mean_rel(o, single) <= 2e-2
+    if splits != "auto":
+        ref = O.attention_full_int8_splitkv(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], False, sm, splits, block_n=128)
+        assert max_abs(o, ref) <= 4e-3 and mean_rel(o, ref) <= 2e-4
+
+
+def test_decode_blocked_v_scales_bf16_and_strided_cache():
+    B, H, H_kv, Nq, Nk, D = 2, 4, 2, 2, 900, 128
+    x = decode_inputs(B, H, H_kv, Nq, Nk, D, seed=92, dtype=torch.bfloat16, v_block=256)
+    sm = D ** -0.5
+    # the cache lives in a longer allocation (row stride unchanged, batch/head strides larger)
+    kbig = torch.zeros((B, H_kv, 1024, D), dtype=torch.int8, device=DEV); kbig[:, :, :Nk] = x["k8"].to(DEV)
+    vbig = torch.zeros((B, H_kv, 1024, D), dtype=torch.int8, device=DEV); vbig[:, :, :Nk] = x["v8"].to(DEV)
+    q8, qs, ks, vs = gpu(x["q8"], x["qs"], x["ks"], x["vs"])
+    o = M.attention_full_int8(q8, kbig[:, :, :Nk], vbig[:, :, :Nk], qs, ks, vs, False, sm, out_dtype=torch.bfloat16,
+                              v_scale_block=256)
+    torch.cuda.synchronize()
+    ref = oracle(x, sm, 128, p_requant=O.p_requant_rne, out_dtype=torch.bfloat16, v_scale_block=256)
+    assert o.dtype == torch.bfloat16
+    assert max_abs(o, ref) <= 3e-2 and mean_rel(o, ref) <= 3e-3            # bf16 output: 8-bit significand
+
+
+def test_decode_kernel_agrees_with_the_general_kernel():
+    """65 query rows run the general kernel, the first 64 of them alone the decode kernel: same rows, same block maxima,
+    same P8 and the same int32 sums, so the outputs differ only through the order of the fp32 row-sum additions."""
+    x = decode_inputs(1, 2, 2, 65, 1500, 128, seed=93)
+    sm = 128 ** -0.5
+    k8, v8, ks, vs = gpu(x["k8"], x["v8"], x["ks"], x["vs"])
+    q8, qs = gpu(x["q8"], x["qs"])
+    general = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm)
+    decode = M.attention_full_int8(q8[:, :, :64].contiguous(), k8, v8, qs[:, :, :64].contiguous(), ks, vs, False, sm)
+    torch.cuda.synchronize()
+    assert max_abs(decode, general[:, :, :64]) <= 1e-3 and mean_rel(decode, general[:, :, :64]) <= 1e-5
+
+
+def test_decode_full_size_against_one_head_of_the_oracle():
+    """The benchmark's decode shape (B8 H32 Nk16384 d128, one query per head): one (batch, head) against the oracle, and
+    the whole output reproducible between two launches."""
+    B, H, Nk, D = 8, 32, 16384, 128
+    g = torch.Generator(device=DEV).manual_seed(94)
+    q8 = torch.randint(-127, 128, (B, H, 1, D), generator=g, device=DEV, dtype=torch.int8)
+    k8 = torch.randint(-127, 128, (B, H, Nk, D), generator=g, device=DEV, dtype=torch.int8)
+    v8 = torch.randint(-127, 128, (B, H, Nk, D), generator=g, device=DEV, dtype=torch.int8)
+    qs = (torch.rand((B, H, 1), generator=g, device=DEV) * 0.01 + 0.02).half()
+    ks = (torch.rand((B, H, Nk), generator=g, device=DEV) * 0.01 + 0.02).half()
+    vs = (torch.rand((B, H), generator=g, device=DEV) * 0.01 + 0.02).half()
+    sm = D ** -0.5
+    o1 = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, num_splits="auto")
+    o2 = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, num_splits="auto")
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2)
+    b, h = 5, 17
+    c = lambda t: t[b:b + 1, h:h + 1].cpu()
+    single = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm)
+    ref = O.attention_full_int8(c(q8), c(k8), c(v8), c(qs), c(ks), c(vs), False, sm, block_n=128, p_requant=O.p_requant_rne)
+    assert max_abs(single[b:b + 1, h:h + 1], ref) <= 2e-3
+    # the split pass quantises P per split (outputs here are of order one: compare in the mean-relative measure)
+    assert mean_rel(o1[b:b + 1, h:h + 1], ref) <= 3e-2

@@ -404,3 +404,17 @@ def test_blocked_v_scale_split_agrees_with_single_pass():
     two = O.attention_full_int8_splitkv(q8, k8, v8, qs, ks, vs, False, 0.2, 2, block_m=64, block_n=64, v_scale_block=64).float()
     # (the second split quantises P against its own maximum: same size of deviation as with a scalar V scale)
     assert (one - two).abs().max() < 3e-2 and (one - two).abs().mean() < 2e-3
+
+
+def test_separate_query_and_key_lengths_are_row_slices_of_the_square_case():
+    q, k, v, _ = O.make_inputs(1, 2, 200, 32, seed=17)
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    square = O.attention_full_int8(q8, k8, v8, qs, ks, vs, False, 0.2, block_m=64, block_n=64)
+    part = O.attention_full_int8(q8[:, :, 70:75], k8, v8, qs[:, :, 70:75], ks, vs, False, 0.2, block_m=64, block_n=64)
+    assert part.shape == (1, 2, 5, 32) and torch.equal(part, square[:, :, 70:75])
+    half = O.attention_int8(q8[:, :, :3], k8, v, qs[:, :, :3], ks, False, 0.2, block_m=64, block_n=64)
+    assert torch.equal(half, O.attention_int8(q8, k8, v, qs, ks, False, 0.2, block_m=64, block_n=64)[:, :, :3])
+    two = O.attention_full_int8_splitkv(q8[:, :, 70:75], k8, v8, qs[:, :, 70:75], ks, vs, False, 0.2, 2, block_m=64, block_n=64)
+    assert torch.equal(two, O.attention_full_int8_splitkv(q8, k8, v8, qs, ks, vs, False, 0.2, 2, block_m=64, block_n=64)[:, :, 70:75])
+    with pytest.raises(AssertionError):
+        O.attention_full_int8(q8[:, :, :5], k8, v8, qs[:, :, :5], ks, vs, True, 0.2, block_m=64, block_n=64)
