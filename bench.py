@@ -38,6 +38,9 @@ WORKLOADS = {
                                               dtype="bfloat16", std=0.5),
     # the headline shape with V quantised per block of 128 keys and channel (the V scales of the reference's CUDA kernel)
     "full_int8_B4_H32_N4096_d128_vblock": dict(variant="full", B=4, H=32, N=4096, D=128, causal=False, splits=1, v_block=128),
+    # decoding against a cache: one query per head, 16384 cached keys (HBM-bound: K and V are streamed once)
+    "full_int8_decode_B8_H32_Nq1_Nk16384_d128": dict(variant="full", B=8, H=32, N=1, Nk=16384, D=128, causal=False, splits="auto"),
+    "full_int8_decode_B32_H32_Nq1_Nk4096_d128": dict(variant="full", B=32, H=32, N=1, Nk=4096, D=128, causal=False, splits=1),
     # the input quantisers (HBM-bound): Q/K per token, V per (batch, head)
     "quant_pertoken_B4_H32_N4096_d128": dict(variant="quant_token", B=4, H=32, N=4096, D=128, causal=False, splits=1),
     "quant_pertensor_B4_H32_N4096_d128": dict(variant="quant_tensor", B=4, H=32, N=4096, D=128, causal=False, splits=1),
@@ -48,6 +51,8 @@ WORKLOADS = {
 MEASURED_TRAFFIC_BYTES = {
     # FETCH_SIZE x 1.9997 + WRITE_SIZE x 1.0 (KiB per dispatch, factors from a 256 MiB copy): 194.2 MiB read + 128 MiB written
     "full_int8_B4_H32_N4096_d128": 337860823,
+    # FETCH_SIZE 528548.6 x 1.9998 + WRITE_SIZE 256 x 1.0: 1032.2 MiB read + 0.25 MiB written (algorithmic: 1082523648)
+    "full_int8_decode_B32_H32_Nq1_Nk4096_d128": 1082610029,
 }
 
 
@@ -140,8 +145,9 @@ def main():
     std = w.get("std", 1.0)
     sm = D ** -0.5
     g = torch.Generator(device=dev).manual_seed(20)
-    mk = lambda: (torch.randn((B, H, N, D), generator=g, device=dev, dtype=torch.float32) * std).to(dt)
-    q, k, v = mk(), mk(), mk()
+    Nk = w.get("Nk", N)
+    mk = lambda n=N: (torch.randn((B, H, n, D), generator=g, device=dev, dtype=torch.float32) * std).to(dt)
+    q, k, v = mk(), mk(Nk), mk(Nk)
     outlier_cols = []
     if w.get("k_outlier_frac"):
         n_out = max(1, round(w["k_outlier_frac"] * D))
@@ -162,7 +168,8 @@ def main():
                                                  p_round=args.p_round, v_scale_block=v_block)
         else:
             step = lambda: M.attention_int8(q8, k8, v, qs, ks, causal, sm, num_splits=splits)
-    ops = ops_of(B, H, N, D, causal)
+    ops = ops_of(B, H, N, D, causal) * (Nk / N)
+    decode = Nk != N
 
     if args.copy_probe_mib > 0:
         src = torch.empty((args.copy_probe_mib << 20,), dtype=torch.uint8, device=dev).random_(0, 255)
@@ -200,13 +207,15 @@ def main():
         if variant == "full":
             a8 = (c(q8), c(k8), c(v8), c(qs), c(ks), c(vs), causal, sm)
             okw = dict(v_scale_block=v_block) if v_block else {}
-            if splits > 1:
+            if splits != "auto" and splits > 1:
                 # a split restarts the running maximum, so its P8 is quantised in another frame than the single pass:
                 # the oracle evaluated with the same split is the reference; the single pass is shown beside it
                 refs["vs_oracle_split_reference_rounding"] = O.attention_full_int8_splitkv(*a8, splits, block_n=bn, out_dtype=dt)
                 refs["vs_single_pass_reference_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt)
             else:
                 refs["vs_reference_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt, **okw)
+            if splits == "auto":
+                refs = {"vs_single_pass_reference_rounding": O.attention_full_int8(*a8, block_n=bn, out_dtype=dt, **okw)}
             if args.p_round == "rne" and splits == 1:
                 refs["vs_same_rounding"] = O.attention_full_int8(*a8, block_n=bn, out_dtype=dt, p_requant=O.p_requant_rne, **okw)
         elif variant == "half":
@@ -246,8 +255,22 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TOP/s" if variant == "full" else "TFLOP/s",
                      "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel": kernel_name, "avg_launch_ms": kern_ms, "peak_model": peak_model,
-                     "launch_includes": "forward kernel" + (" + split-KV combine kernel" if splits > 1 else "")},
+                     "launch_includes": "forward kernel" + (" + split-KV combine kernel" if splits != 1 else "")},
     }
+    if decode:
+        # one pass over the cached K and V (int8) and their scales; Q, O and the split partials are a rounding error
+        sb = 2 if dt != torch.float32 else 4
+        alg_bytes = B * H * Nk * (2 * D + sb) + B * H * N * D * 3
+        gbs = alg_bytes / (kern_ms * 1e-3) / 1e9
+        out["metric"] = "decode attention: cached K+V bytes streamed per second (full-int8, one query per head)"
+        out["value"], out["unit"] = alg_bytes / (ms_step * 1e-3) / 1e9, "GB/s"
+        out["config"]["seqlen_k"] = Nk
+        out["config"]["bytes_per_step"] = alg_bytes
+        out.pop("pct_int8_peak")
+        out["roofline"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                           "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "fwd_decode_full_int8_kernel",
+                           "avg_launch_ms": kern_ms,
+                           "launch_includes": "forward kernel" + (" + split-KV combine kernel" if splits != 1 else "")}
     if parity is not None:
         out["parity"] = parity
     if args.cpu_seconds > 0:
