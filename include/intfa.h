@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define INTFA_VERSION 3
+#define INTFA_VERSION 4
 
 /* forward variants (one entry point each, below) */
 enum { INTFA_VARIANT_FULL_INT8 = 0, INTFA_VARIANT_HALF_INT8 = 1, INTFA_VARIANT_FP16 = 2 };
@@ -49,7 +49,7 @@ enum {
     INTFA_OK = 0,
     INTFA_ERR_NULL = -1,          /* a required pointer is NULL */
     INTFA_ERR_HEAD_DIM = -2,      /* head_dim not supported by the kernels */
-    INTFA_ERR_SEQLEN = -3,        /* seqlen not positive, or causal with seqlen_k != seqlen */
+    INTFA_ERR_SEQLEN = -3,        /* seqlen not positive, or causal with seqlen_k != seqlen or with seqlens_k */
     INTFA_ERR_ALIGN = -4,         /* pointer or row stride not 16-byte aligned */
     INTFA_ERR_DTYPE = -5,         /* unknown dtype enum */
     INTFA_ERR_WORKSPACE = -6,     /* workspace missing or too small for the requested split count */
@@ -119,6 +119,11 @@ typedef struct intfa_fwd_params {
                                  intfa_fwd_block_n(INTFA_VARIANT_FULL_INT8, head_dim). */
     int32_t reserved0;        /* set to 0 */
     int64_t vs_stride_blk;    /* elements between consecutive scale rows of v_scale (>= head_dim) */
+    const int32_t* seqlens_k; /* optional device array [batch]: number of keys of each batch entry, 0 <= n <= seqlen_k (a
+                                 key/value cache filled to different lengths; the counterpart of the reference's
+                                 cu_seqlens_k used as lengths / seqused_k, csrc/flash.h:95-99,149-151, csrc/block_info.h:21-22).  k, v and k_scale keep their seqlen_k-row
+                                 layout; rows past a batch entry's length are not read.  An entry with no key gives zeros
+                                 (lse = -inf).  NULL = every entry has seqlen_k keys.  Not with causal. */
 } intfa_fwd_params;
 
 /* Library/ABI version (INTFA_VERSION of the build). */

@@ -56,7 +56,7 @@ def _require_gpu(*ts):
 
 def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float, out_dtype,
                    num_splits: int = 1, p_round: int = _capi.PROUND_RNE, return_lse: bool = False,
-                   v_scale_block: Optional[int] = None):
+                   v_scale_block: Optional[int] = None, seqlens_k: Optional[torch.Tensor] = None):
     lib = _capi.load()
     _require_gpu(q, k, v, q_scale, k_scale, v_scale)
     d = check_head_dims(q, k, v)
@@ -114,6 +114,16 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
     p.batch, p.heads, p.seqlen, p.head_dim = Z, H, N, dk
     p.heads_kv = H_kv
     p.seqlen_k = N_k
+    if seqlens_k is not None:
+        # number of keys per batch entry (a cache filled to different lengths); int32 [Z] on the device
+        _require_gpu(seqlens_k)
+        if causal:
+            raise ValueError("per-batch key lengths are for non-causal attention (decoding against a cache)")
+        if seqlens_k.dtype != torch.int32 or tuple(seqlens_k.shape) != (Z,):
+            raise ValueError(f"seqlens_k must be an int32 tensor of shape ({Z},)")
+        seqlens_k = seqlens_k.contiguous()
+        p.seqlens_k = seqlens_k.data_ptr()
+        keep.append(seqlens_k)
     # Few queries per head with grouped K/V heads (decoding): the g query heads of a group become g*N rows of ONE head,
     # so that a group streams its K/V once instead of g times.  Pure re-striding: same memory, same results per row.
     g = H // H_kv

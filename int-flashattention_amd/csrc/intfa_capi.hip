@@ -77,6 +77,11 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
         }
     }
     k.lse = p->lse;
+    if (p->seqlens_k != nullptr) {
+        if (p->causal) return INTFA_ERR_SEQLEN;                              // as seqlen_k: no causal mask over two lengths
+        if (reinterpret_cast<uintptr_t>(p->seqlens_k) & 3u) return INTFA_ERR_ALIGN;
+        k.seqlens_k = p->seqlens_k;
+    }
     k.batch = p->batch; k.heads = p->heads; k.seqlen = p->seqlen; k.seqlen_k = seqlen_k; k.head_dim = p->head_dim;
     k.scale_dtype = p->scale_dtype; k.causal = p->causal ? 1 : 0;
     k.kv_group = p->heads / heads_kv;

@@ -45,6 +45,7 @@ struct KParams {
     const char* q; const char* k; const char* v; char* out;
     const char* q_scale; const char* k_scale; const char* v_scale;
     float* lse;
+    const int32_t* seqlens_k;              // optional [batch]: number of keys per batch entry (<= seqlen_k)
     int32_t* s_dump;                       // debug: int32 S [B,H,N,N]
     float* o_part; float* lse_part;        // split-KV partials [S,B,H,N,D] fp32 / [S,B,H,N]
     int64_t q_sb, q_sh, q_sn;              // bytes

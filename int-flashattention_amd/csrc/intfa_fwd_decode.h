@@ -74,7 +74,13 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const int b = head / p.heads, h = head % p.heads;
     const int hk = h / kv_group;
 
-    const int nb_total = (p.seqlen_k + BN - 1) / BN;
+    // number of keys of this batch entry: one length for all, or per batch (a cache filled to different lengths)
+    int seqlen_k = p.seqlen_k;
+    if (p.seqlens_k != nullptr) {            // clamped to [0, seqlen_k]: rows past the allocation are never addressed
+        const int n = p.seqlens_k[b];
+        seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
+    }
+    const int nb_total = (seqlen_k + BN - 1) / BN;
     int nb_begin = 0, nb_end = nb_total;
     if (SPLIT) {                                           // csrc/flash_fwd_kernel.h:503-511
         nb_begin = split * p.blocks_per_split;
@@ -105,8 +111,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     // ---- global -> LDS copies (asynchronous, straight into LDS; the four waves split the instructions)
     const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
     const char* Vg = p.v + b * p.v_sb + hk * p.v_sh;
-    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen_k - 1) * p.k_sn + D));
-    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen_k - 1) * p.v_sn + D));
+    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((seqlen_k - 1) * p.k_sn + D));
+    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((seqlen_k - 1) * p.v_sn + D));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
     const auto k_lane = tile_load_lane<D, SWZ_K, BN>(k_sn, wave, lane);
     const auto v_lane = tile_load_lane<D, SWZ_V8, BN>(v_sn, wave, lane);
@@ -121,7 +127,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const int ks_stride = (int)(p.ks_sn * ks_esize);
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
         int key = nb * BN + (tid & (BN - 1));
-        key = key < p.seqlen_k ? key : p.seqlen_k - 1;                  // keys past the end are masked later
+        key = key < seqlen_k ? key : seqlen_k - 1;                  // keys past the end are masked later
         const char* src = Ksg + (int64_t)key * ks_stride;
         if (p.scale_dtype == 2) return *(const uint32_t*)src;
         return (uint32_t)*(const uint16_t*)src;
@@ -167,7 +173,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const uint32_t vs_wr = OFF_VS + 4 * (vs_thread ? vs_c : 0);
     const uint32_t vs_rd = OFF_VS + 16 * lh;                         // + 4 * (32*dt + 8*a4) per read
     const bool own_tile0 = wave < DT;                                // head_dim 64: waves 2 and 3 own no output tile
-    const int tail_keys = p.seqlen_k - (nb_total - 1) * BN;          // valid keys of the last block
+    const int tail_keys = seqlen_k - (nb_total - 1) * BN;          // valid keys of the last block
 
     auto step = [&](auto buf_tag, int nb) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
@@ -297,10 +303,10 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const float l_tot = (*(const float*)(smem + xm_rd) + *(const float*)(smem + xm_rd + 128)) +
                         (*(const float*)(smem + xm_rd + 256) + *(const float*)(smem + xm_rd + 384));   // units of 1/127 when PROUND == 0
     const float vs = VBLK ? 1.f : load_scale(p.v_scale, b * p.vs_sb + hk * p.vs_sh, p.scale_dtype);
-    const float out_scale = (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
+    const bool seen = nb_begin < nb_end;         // false: an empty split range, or an empty cache entry (zeros, lse = -inf)
+    const float out_scale = !seen ? 0.f : (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
     const float l_true = (PROUND == 0) ? l_tot * (1.f / 127.f) : l_tot;
-    const float lse = m_run + __builtin_log2f(l_true);
-    const bool seen = nb_begin < nb_end;
+    const float lse = seen ? m_run + __builtin_log2f(l_true) : -INFINITY;
     if (!q_valid) return;
     if (SPLIT) {
         const int64_t row = ((int64_t)(split * p.batch + b) * p.heads + h) * p.seqlen + q_row;

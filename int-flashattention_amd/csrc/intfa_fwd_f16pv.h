@@ -91,7 +91,13 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     const int hk = h / kv_group;                     // K/V head of this query head
     // ragged sequence lengths are handled as in the full-int8 kernel (zero-filled copies, masked last block, rows past
     // the end computed on clamped inputs and not stored)
-    const int nb_total = (p.seqlen_k + BN - 1) / BN;
+    // number of keys of this batch entry: one length for all, or per batch (a cache filled to different lengths)
+    int seqlen_k = p.seqlen_k;
+    if (p.seqlens_k != nullptr) {            // clamped to [0, seqlen_k]: rows past the allocation are never addressed
+        const int n = p.seqlens_k[b];
+        seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
+    }
+    const int nb_total = (seqlen_k + BN - 1) / BN;
     int nb_begin = 0, nb_end = CAUSAL ? ((mb + 1) * RDIAG < nb_total ? (mb + 1) * RDIAG : nb_total) : nb_total;
     if (SPLIT) {
         // non-causal: the key blocks of the sequence are dealt evenly to the splits (csrc/flash_fwd_kernel.h:503-511);
@@ -125,8 +131,8 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     // ---- global -> LDS copies
     const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
     const char* Vg = p.v + b * p.v_sb + hk * p.v_sh;
-    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen_k - 1) * p.k_sn + KROW));
-    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen_k - 1) * p.v_sn + VROW));
+    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((seqlen_k - 1) * p.k_sn + KROW));
+    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((seqlen_k - 1) * p.v_sn + VROW));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
     const auto k_lane = tile_load_lane<KROW, SWZ_K, BN>(k_sn, wave, lane);
     const auto v_lane = tile_load_lane<VROW, SWZ_V16, BN>(v_sn, wave, lane);
@@ -141,7 +147,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
         if (!QK_INT8 || tid >= BN) return 0u;
         int key = nb * BN + tid;
-        key = key < p.seqlen_k ? key : p.seqlen_k - 1;                                    // keys past the end are masked later
+        key = key < seqlen_k ? key : seqlen_k - 1;                                    // keys past the end are masked later
         const char* src = Ksg + (int64_t)key * ks_stride;
         if (p.scale_dtype == 2) return *(const uint32_t*)src;
         return (uint32_t)*(const uint16_t*)src;
@@ -324,7 +330,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
             if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
         }
         const int diag_begin = mb * RDIAG;
-        const int tail_keys = p.seqlen_k - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
+        const int tail_keys = seqlen_k - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
         const bool ragged = !CAUSAL && tail_keys < BN && nb_end == nb_total;
         const int plain_end = CAUSAL ? (nb_end > diag_begin ? diag_begin : nb_end) : (ragged ? nb_end - 1 : nb_end);
         int nb = nb_begin;
@@ -352,8 +358,10 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     const int e_heads = pe->heads, e_seqlen = pe->seqlen;
     const int eb = head / e_heads, eh = head % e_heads;
     const float l_tot = half_pair_sum(l_run);
-    const float inv = 1.f / l_tot;
-    const float lse = m_run + __builtin_log2f(l_tot);
+    // (no key at all - an empty cache entry - gives zeros and lse = -inf instead of 0 / 0)
+    const bool any_key = nb_begin < nb_end;
+    const float inv = any_key ? 1.f / l_tot : 0.f;
+    const float lse = any_key ? m_run + __builtin_log2f(l_tot) : -INFINITY;
     if (SPLIT) {
         const int64_t row = ((int64_t)(split * pe->batch + eb) * e_heads + eh) * e_seqlen + q_row;
         float* op = pe->o_part + row * D;

@@ -104,7 +104,13 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     // Sequence lengths that are not a multiple of the block sizes: the copies of K/V rows past the end return zeros
     // (bounds-checked buffer loads), the last key block runs the masked code instance, query rows past the end are
     // computed on clamped inputs and not stored.
-    const int nb_total = (p.seqlen_k + BN - 1) / BN;
+    // number of keys of this batch entry: one length for all, or per batch (a cache filled to different lengths)
+    int seqlen_k = p.seqlen_k;
+    if (p.seqlens_k != nullptr) {            // clamped to [0, seqlen_k]: rows past the allocation are never addressed
+        const int n = p.seqlens_k[b];
+        seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
+    }
+    const int nb_total = (seqlen_k + BN - 1) / BN;
     int nb_begin = 0, nb_end = CAUSAL ? ((mb + 1) * RDIAG < nb_total ? (mb + 1) * RDIAG : nb_total) : nb_total;
     if (SPLIT) {
         // non-causal: the key blocks of the sequence are dealt evenly to the splits (csrc/flash_fwd_kernel.h:503-511);
@@ -138,8 +144,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     // ---- global -> LDS copies (asynchronous, straight into LDS)
     const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
     const char* Vg = DUMP_S ? Kg : p.v + b * p.v_sb + hk * p.v_sh + half * DV;
-    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((p.seqlen_k - 1) * p.k_sn + D));
-    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((p.seqlen_k - 1) * p.v_sn + DV));
+    const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((seqlen_k - 1) * p.k_sn + D));
+    const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((seqlen_k - 1) * p.v_sn + DV));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
     const auto k_lane = tile_load_lane<D, SWZ_K, BN>(k_sn, wave, lane);
     const auto v_lane = tile_load_lane<DV, SWZ_V8, BN>(v_sn, wave, lane);
@@ -174,7 +180,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {           // raw bits
         if (DUMP_S) return 0u;
         int key = nb * BN + ks_key;
-        key = key < p.seqlen_k ? key : p.seqlen_k - 1;                                    // keys past the end are masked later
+        key = key < seqlen_k ? key : seqlen_k - 1;                                    // keys past the end are masked later
         const char* src = Ksg + (int64_t)key * ks_stride;
         if (p.scale_dtype == 2) return *(const uint32_t*)src;
         return (uint32_t)*(const uint16_t*)src;
@@ -453,7 +459,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             if (vs_thread) *(float*)(smem + vs_wr) = load_vs(nb_begin);
         }
         const int diag_begin = mb * RDIAG;                 // first key block that touches the diagonal
-        const int tail_keys = p.seqlen_k - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
+        const int tail_keys = seqlen_k - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
         const bool ragged = !CAUSAL && tail_keys < BN && nb_end == nb_total;
         const int plain_end = CAUSAL ? (nb_end > diag_begin ? diag_begin : nb_end) : (ragged ? nb_end - 1 : nb_end);
         int nb = nb_begin;
@@ -485,9 +491,11 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     const int eb = head / e_heads, eh = head % e_heads;
     const float l_tot = half_pair_sum(l_run);          // in units of 1/127 when PROUND == 0
     const float vs = VBLK ? 1.f : load_scale(pe->v_scale, eb * pe->vs_sb + (eh / pe->kv_group) * pe->vs_sh, pe->scale_dtype);
-    const float out_scale = (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
+    // (no key at all - an empty cache entry - gives zeros and lse = -inf instead of 0 / 0)
+    const bool any_key = nb_begin < nb_end;
+    const float out_scale = !any_key ? 0.f : (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
     const float l_true = (PROUND == 0) ? l_tot * (1.f / 127.f) : l_tot;
-    const float lse = m_run + __builtin_log2f(l_true);
+    const float lse = any_key ? m_run + __builtin_log2f(l_true) : -INFINITY;
     if (SPLIT) {
         const int64_t row = ((int64_t)(split * pe->batch + eb) * e_heads + eh) * e_seqlen + q_row;
         float* op = pe->o_part + row * D + half * DV;

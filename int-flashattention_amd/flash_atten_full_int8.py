@@ -6,7 +6,7 @@ from ._host import launch_forward
 
 
 def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, *, out_dtype=torch.float16,
-                        num_splits=1, p_round="rne", return_lse=False, v_scale_block=None):
+                        num_splits=1, p_round="rne", return_lse=False, v_scale_block=None, seqlens_k=None):
     """Full-int8 attention forward.
 
     q, k, v: int8 [Z, H, N, d]; q_scale, k_scale: [Z, H, N] per-token scales; v_scale: [Z, H];
@@ -20,9 +20,13 @@ def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, *,
     ``quant_perblock_channel``.  ``v_scale_block`` defaults to the kernel's key-block length (``block_n("full", d)``)
     and must be a multiple of it.
 
+    ``seqlens_k`` (int32 [Z] on the device, non-causal only): number of keys of each batch entry when k and v are a cache
+    filled to different lengths; rows past an entry's length are not read.
+
     ``p_round``: "rne" folds 127 into the exponent and rounds to nearest-even; "reference" reproduces the
     fp16 sequence of flash_atten_full_int8.py:49-51.
     """
     pr = {"rne": _capi.PROUND_RNE, "reference": _capi.PROUND_REFERENCE}[p_round]
     return launch_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, out_dtype,
-                          num_splits=num_splits, p_round=pr, return_lse=return_lse, v_scale_block=v_scale_block)
+                          num_splits=num_splits, p_round=pr, return_lse=return_lse, v_scale_block=v_scale_block,
+                          seqlens_k=seqlens_k)

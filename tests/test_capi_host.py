@@ -83,6 +83,8 @@ def _valid_block():
     (lambda p: (setattr(p, "v_scale_block", 64), setattr(p, "vs_stride_blk", 128)), -9),    # not a multiple of the key block (128)
     (lambda p: (setattr(p, "v_scale_block", 128), setattr(p, "vs_stride_blk", 64)), -9),    # scale rows overlap
     (lambda p: setattr(p, "v_scale_block", -1), -9),
+    (lambda p: (setattr(p, "causal", 1), setattr(p, "seqlens_k", 0x10000)), -3),        # per-batch key lengths are non-causal
+    (lambda p: setattr(p, "seqlens_k", 0x10002), -4),
     (lambda p: (setattr(p, "v_scale_block", 128), setattr(p, "vs_stride_blk", 128), setattr(p, "v_scale", 0x10002)), -4),
 ])
 def test_validation_rejects_bad_blocks_before_touching_the_gpu(mutate, code):

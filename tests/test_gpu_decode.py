@@ -122,3 +122,63 @@ def test_decode_full_size_against_one_head_of_the_oracle():
     assert max_abs(single[b:b + 1, h:h + 1], ref) <= 2e-3
     # the split pass quantises P per split (outputs here are of order one: compare in the mean-relative measure)
     assert mean_rel(o1[b:b + 1, h:h + 1], ref) <= 3e-2
+
+
+# ------------------------------------------------------------------------------------------ per-batch key lengths
+@pytest.mark.parametrize("variant,Nq,D", [("full", 1, 128), ("full", 40, 64), ("full", 200, 128), ("half", 3, 128), ("fp", 130, 64)])
+def test_per_batch_key_lengths_equal_sliced_calls(variant, Nq, D):
+    """k and v are a cache filled to different lengths per batch entry: every entry must come out exactly as a call on
+    that entry alone with the cache sliced to its length (same kernels, same blocks: bit for bit), and an empty entry as
+    zeros with lse = -inf."""
+    B, H, Nk = 4, 2, 700
+    lens = [700, 129, 0, 1]
+    x = decode_inputs(B, H, H, Nq, Nk, D, seed=95)
+    sm = D ** -0.5
+    sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
+
+    def call(sel_b, nk, **kw):
+        c = lambda t: t[sel_b].to(DEV)
+        if variant == "full":
+            return M.attention_full_int8(c(x["q8"]), c(x["k8"])[:, :, :nk], c(x["v8"])[:, :, :nk], c(x["qs"]), c(x["ks"])[:, :, :nk],
+                                         c(x["vs"]), False, sm, return_lse=True, **kw)
+        if variant == "half":
+            return M.attention_int8(c(x["q8"]), c(x["k8"])[:, :, :nk], c(x["v"])[:, :, :nk], c(x["qs"]), c(x["ks"])[:, :, :nk],
+                                    False, sm, return_lse=True, **kw)
+        return M.attention(c(x["q"]), c(x["k"])[:, :, :nk], c(x["v"])[:, :, :nk], False, sm, return_lse=True, **kw)
+
+    o, lse = call(slice(None), Nk, seqlens_k=sl)
+    torch.cuda.synchronize()
+    assert o.shape == (B, H, Nq, D) and torch.isfinite(o).all()
+    for b, n in enumerate(lens):
+        if n == 0:
+            assert o[b].abs().max().item() == 0 and torch.isinf(lse[b]).all() and (lse[b] < 0).all()
+            continue
+        ob, lb = call(slice(b, b + 1), n)
+        assert torch.equal(o[b:b + 1], ob) and torch.equal(lse[b:b + 1], lb), f"batch entry {b} (length {n})"
+
+
+def test_per_batch_key_lengths_with_split_kv_and_argument_checks():
+    B, H, Nq, Nk, D = 3, 4, 2, 1500, 128
+    lens = [1500, 300, 77]
+    x = decode_inputs(B, H, H, Nq, Nk, D, seed=96)
+    sm = D ** -0.5
+    args = gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"])
+    sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    one = M.attention_full_int8(*args, False, sm, seqlens_k=sl, p_round="reference")
+    split = M.attention_full_int8(*args, False, sm, seqlens_k=sl, num_splits=4, p_round="reference")   # some splits of short entries are empty
+    torch.cuda.synchronize()
+    assert torch.isfinite(split).all()
+    for b, n in enumerate(lens):
+        c = lambda t: t[b:b + 1]
+        ref = O.attention_full_int8(c(x["q8"]), c(x["k8"])[:, :, :n], c(x["v8"])[:, :, :n], c(x["qs"]), c(x["ks"])[:, :, :n],
+                                    c(x["vs"]), False, sm, block_n=128)
+        assert max_abs(one[b:b + 1], ref) <= 4e-3
+        assert max_abs(split[b:b + 1], ref) <= MAX_ABS and mean_rel(split[b:b + 1], ref) <= 3e-2
+    with pytest.raises(ValueError):
+        M.attention_full_int8(*args, False, sm, seqlens_k=sl.long())
+    with pytest.raises(ValueError):
+        M.attention_full_int8(*args, False, sm, seqlens_k=sl[:2])
+    sq = decode_inputs(1, 2, 2, 128, 128, 64, seed=97)
+    with pytest.raises(ValueError):
+        M.attention_full_int8(*gpu(sq["q8"], sq["k8"], sq["v8"], sq["qs"], sq["ks"], sq["vs"]), True, 0.1,
+                              seqlens_k=torch.tensor([128], dtype=torch.int32, device=DEV))
