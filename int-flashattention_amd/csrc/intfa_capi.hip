@@ -126,9 +126,11 @@ int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t str
 
 // Few query rows per head and no causal mask (decoding against a cache): the full-int8 pass runs the kernel whose waves
 // share the keys of a block instead of each taking 32 query rows.
+// (Head_dim 256 stays with the general kernel: its key block is 64 there, the decode kernel's is 128, and the block
+// length is part of the arithmetic that intfa_fwd_block_n() promises.)
 constexpr int kDecodeMaxRows = 2 * kDecodeRows;
-bool decode_shaped(int variant, int seqlen, int causal) {
-    return variant == INTFA_VARIANT_FULL_INT8 && !causal && seqlen <= kDecodeMaxRows;
+bool decode_shaped(int variant, int seqlen, int causal, int head_dim) {
+    return variant == INTFA_VARIANT_FULL_INT8 && !causal && seqlen <= kDecodeMaxRows && head_dim <= 128;
 }
 
 int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dump_s, hipStream_t stream) {
@@ -140,10 +142,9 @@ int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dum
     sel.split = kp.num_splits > 1;
     sel.dump_s = dump_s;
     const int d = kp.head_dim;
-    if (!dump_s && decode_shaped(variant, kp.seqlen, kp.causal)) {
+    if (!dump_s && decode_shaped(variant, kp.seqlen, kp.causal, d)) {
         if (d == 64) return launch_decode_full_int8_d64(kp, sel, stream);
         if (d == 128) return launch_decode_full_int8_d128(kp, sel, stream);
-        if (d == 256) return launch_decode_full_int8_d256(kp, sel, stream);
     } else if (vblk) {
         if (d == 64) return launch_full_int8_vblk_d64(kp, sel, stream);
         if (d == 128) return launch_full_int8_vblk_d128(kp, sel, stream);
@@ -216,7 +217,7 @@ int intfa_fwd_suggest_splits(const intfa_fwd_params* p, int variant, int num_cus
     const int cus = num_cus > 0 ? num_cus : 256;
     const int64_t slots = 2ll * cus;                                           // two workgroups per compute unit
     int64_t wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kBlockM - 1) / kBlockM);
-    if (decode_shaped(variant, p->seqlen, p->causal)) wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kDecodeRows - 1) / kDecodeRows);
+    if (decode_shaped(variant, p->seqlen, p->causal, p->head_dim)) wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kDecodeRows - 1) / kDecodeRows);
     else if (variant == INTFA_VARIANT_FULL_INT8 && p->head_dim == 256) wgs *= 2;     // column halves
     if (wgs * 5 >= slots * 4) return 1;                                        // at least 80 % of the slots are used anyway
     const int seqlen_k = p->seqlen_k > 0 ? p->seqlen_k : p->seqlen;

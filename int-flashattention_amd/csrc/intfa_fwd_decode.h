@@ -20,8 +20,10 @@ namespace intfa {
 
 constexpr int kDecodeRows = 32;       // query rows per workgroup of the decode kernel
 
+// Head dims 64 and 128 (the key block of the general kernel is 128 there too, so both kernels evaluate the same blocks).
 template <int D, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool SPLIT, bool VBLK>
 __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const KParams p) {
+    static_assert(D == 64 || D == 128, "the decode kernel shares the 128-key block of the general kernel");
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T
     constexpr int DT = D / 32;                   // 32-wide output tiles along head_dim; wave w owns tiles w, w+4, ...
@@ -137,8 +139,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
         if (p.scale_dtype == 1) return __builtin_bit_cast(float, raw << 16);
         return __builtin_bit_cast(float, raw);
     };
-    // VBLK: fp32 channel scales of a key block; thread 128 + c fetches channel c (D = 256: threads 0 .. 255)
-    const int vs_c = D <= 128 ? tid - 128 : tid;
+    // VBLK: fp32 channel scales of a key block; thread 128 + c fetches channel c
+    const int vs_c = tid - 128;
     const bool vs_thread = VBLK && vs_c >= 0 && vs_c < D;
     const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + (vs_thread ? vs_c : 0));
     auto load_vs = [&](int nb) __attribute__((always_inline)) -> float {

@@ -30,7 +30,6 @@ INTFA_DECL_LAUNCH(launch_full_int8_vblk_d128);
 INTFA_DECL_LAUNCH(launch_full_int8_vblk_d256);
 INTFA_DECL_LAUNCH(launch_decode_full_int8_d64);    // few query rows per head: the waves of a workgroup share the keys
 INTFA_DECL_LAUNCH(launch_decode_full_int8_d128);
-INTFA_DECL_LAUNCH(launch_decode_full_int8_d256);
 INTFA_DECL_LAUNCH(launch_half_int8_d64);
 INTFA_DECL_LAUNCH(launch_half_int8_d128);
 INTFA_DECL_LAUNCH(launch_half_int8_d256);
