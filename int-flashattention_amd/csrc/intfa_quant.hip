@@ -33,28 +33,38 @@ __device__ __forceinline__ uint32_t abs_bits(uint16_t b) { return b & 0x7fffu; }
 struct RowDivisor { float scale, recip; };
 __device__ __forceinline__ RowDivisor make_divisor(float scale) { return {scale, 1.0f / scale}; }
 
-// round(x / scale) truncated to int8, both operands and the quotient in the 16-bit type
-template <int DT> __device__ __forceinline__ int quant_one(uint16_t xb, RowDivisor d) {
+// Round-half-even of four quotients |q| < 128.5 to int8, packed into one word.  Adding 1.5 * 2^23 rounds to an integer
+// in the adder (one unit in the last place of that binade is 1) and leaves the two's-complement byte in the low byte of
+// the bit pattern; two byte permutes and an OR gather the four low bytes.  A NaN (0 / 0: a row or column of zeros has
+// scale 0) keeps a zero low byte, so such elements quantise to 0 without a test per element.
+constexpr float kRoundMagic = 12582912.0f;      // 1.5 * 2^23
+__device__ __forceinline__ uint32_t pack4_rne(float q0, float q1, float q2, float q3) {
+    const uint32_t b0 = __builtin_bit_cast(uint32_t, q0 + kRoundMagic), b1 = __builtin_bit_cast(uint32_t, q1 + kRoundMagic);
+    const uint32_t b2 = __builtin_bit_cast(uint32_t, q2 + kRoundMagic), b3 = __builtin_bit_cast(uint32_t, q3 + kRoundMagic);
+    // v_perm_b32: selector bytes 0-3 pick from the second operand, 4-7 from the first, 0x0c yields zero
+    return __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
+}
+
+// x / scale rounded to the 16-bit type (both operands are values of that type), as a float
+template <int DT> __device__ __forceinline__ float quotient16(uint16_t xb, RowDivisor d) {
     const float x = to_f32<DT>(xb);
     const float q0 = x * d.recip;
     const float e = __builtin_fmaf(-q0, d.scale, x);
     const float q = __builtin_fmaf(e, d.recip, q0);
-    const float r = __builtin_rintf(to_f32<DT>(from_f32<DT>(q)));
-    return (__builtin_fabsf(r) < 2147483648.0f) ? (int)r : 0;                   // NaN / infinity (zero scale) -> 0
+    return to_f32<DT>(from_f32<DT>(q));
 }
 
 template <int DT> __device__ __forceinline__ void quant_store8(const v4i raw, RowDivisor scale, char* dst) {
     int out[2];
 #pragma unroll
     for (int w = 0; w < 2; ++w) {
-        uint32_t pk = 0;
+        float q[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const uint32_t word = (uint32_t)raw[2 * w + j / 2];
-            const uint16_t xb = (uint16_t)(j & 1 ? word >> 16 : word & 0xffffu);
-            pk |= ((uint32_t)quant_one<DT>(xb, scale) & 0xffu) << (8 * j);
+            q[j] = quotient16<DT>((uint16_t)(j & 1 ? word >> 16 : word & 0xffffu), scale);
         }
-        out[w] = (int)pk;
+        out[w] = (int)pack4_rne(q[0], q[1], q[2], q[3]);
     }
     *(v2i*)dst = (v2i){out[0], out[1]};
 }
@@ -79,7 +89,7 @@ struct QuantParams {
 };
 
 // ---- per token: LPR = d / 8 lanes per row, reduction of the row maximum inside those lanes
-constexpr int kRowsInFlight = 4;    // independent 16-byte loads a lane has in flight (HBM latency x bandwidth needs several)
+constexpr int kRowsInFlight = 8;    // independent 16-byte loads a lane has in flight (HBM latency x bandwidth needs several)
 
 // rows are numbered (batch, head, position) in that order; the count fits 31 bits (checked on the host), so the index
 // arithmetic is 32-bit
@@ -212,9 +222,15 @@ template <int DT, int LPR> __global__ void __launch_bounds__(256) quant_blockcha
 #pragma unroll
     for (int j = 0; j < 8; ++j) atomicMax(&smax[sub * 8 + j], m[j]);
     __syncthreads();
-    float sc[8];
+    float sc[8], rc[8];
+    bool plain_division = false;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) sc[j] = to_f32<DT>((uint16_t)smax[sub * 8 + j]) / 127.0f;
+    for (int j = 0; j < 8; ++j) {
+        sc[j] = to_f32<DT>((uint16_t)smax[sub * 8 + j]) / 127.0f;
+        rc[j] = 1.0f / sc[j];
+        // the reciprocal-based quotient below is correctly rounded unless the divisor's significand is all ones
+        plain_division |= (__builtin_bit_cast(uint32_t, sc[j]) & 0x7fffffu) == 0x7fffffu;
+    }
     if (rl == 0) {
         float* dst = scale_out + ((int64_t)bh * nblk + blk) * p.head_dim + sub * 8;
         *(v4f*)dst = (v4f){sc[0], sc[1], sc[2], sc[3]};
@@ -235,16 +251,18 @@ template <int DT, int LPR> __global__ void __launch_bounds__(256) quant_blockcha
             int out[2];
 #pragma unroll
             for (int w2 = 0; w2 < 2; ++w2) {
-                uint32_t pk = 0;
+                float q[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t word = (uint32_t)raw[u][2 * w2 + j / 2];
                     const float x = to_f32<DT>((uint16_t)(j & 1 ? word >> 16 : word & 0xffffu));
-                    const float s = sc[4 * w2 + j];
-                    const int q = s > 0.f ? (int)__builtin_rintf(x / s) : 0;        // IEEE division, round-half-even
-                    pk |= ((uint32_t)q & 0xffu) << (8 * j);
+                    const float s = sc[4 * w2 + j], r = rc[4 * w2 + j];
+                    // RN(x / s) as in quotient16 (0 / 0 = NaN -> 0 below); IEEE division for the exceptional divisor
+                    const float q0 = x * r;
+                    const float e = __builtin_fmaf(-q0, s, x);
+                    q[j] = plain_division ? x / s : __builtin_fmaf(e, r, q0);
                 }
-                out[w2] = (int)pk;
+                out[w2] = (int)pack4_rne(q[0], q[1], q[2], q[3]);
             }
             *(v2i*)(qbase + (int64_t)n * p.head_dim) = (v2i){out[0], out[1]};
         }

@@ -137,3 +137,20 @@ def test_blocked_v_scale_small_head_dim_and_argument_checks():
         M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"][:, :, :1]), False, 0.2, v_scale_block=128)
     with pytest.raises(ValueError):
         M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"][:, :, 0, 0]), False, 0.2, v_scale_block=128)
+
+
+def test_quant_perblock_channel_bit_exact_on_many_magnitudes():
+    """2 M elements whose columns span eight orders of magnitude: the reciprocal-based quotient of the kernel must round
+    like the oracle's division everywhere (ties included: multiples of 1/254 of a column maximum are planted)."""
+    g = torch.Generator().manual_seed(72)
+    x = torch.randn((2, 2, 4096, 128), generator=g)
+    x = x * torch.pow(10.0, torch.rand((1, 1, 1, 128), generator=g) * 8 - 5)
+    x = x.half()
+    col_max = x[:, :, :128].abs().amax(dim=2, keepdim=True).float()
+    ties = (torch.arange(128).view(1, 1, 128, 1).float() + 0.5) / 127.0 * col_max        # exact .5 quotients where representable
+    x[:, :, 1:129:2] = ties[:, :, 1::2].half()
+    q_ref, s_ref = O.quant_perblock_channel(x, 128)
+    q, s = M.quant_perblock_channel(x.to(DEV), 128)
+    torch.cuda.synchronize()
+    assert torch.equal(s.cpu(), s_ref)
+    assert torch.equal(q.cpu(), q_ref)
