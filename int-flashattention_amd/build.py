@@ -18,6 +18,24 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+C_CALLER_SRC = os.path.join(os.path.dirname(HERE), "tests", "capi_c", "intfa_c_caller.c")
+C_CALLER = C_CALLER_SRC[:-2]
+
+
+def build_c_caller(verbose: bool = True) -> str:
+    """Compiles the plain-C caller of the ABI (tests/capi_c) with gcc against include/intfa.h and libintfa.so."""
+    root = os.path.dirname(HERE)
+    cmd = ["gcc", "-std=c11", "-O2", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(root, "include"), "-I", "/opt/rocm/include",
+           C_CALLER_SRC, "-o", C_CALLER, "-L", HERE, "-lintfa", "-L", "/opt/rocm/lib", "-lamdhip64", "-lm",
+           "-Wl,-rpath,$ORIGIN/../../int-flashattention_amd", "-Wl,-rpath,/opt/rocm/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"gcc failed for {C_CALLER_SRC}:\n{r.stderr[-4000:]}")
+    if verbose:
+        print(f"built {C_CALLER}")
+    return C_CALLER
+
+
 def build(verbose: bool = True, jobs: int = 8) -> str:
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
@@ -39,6 +57,8 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
         raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
     if verbose:
         print(f"built {OUT} from {len(srcs)} source file(s)")
+    if os.path.exists(C_CALLER_SRC):
+        build_c_caller(verbose)
     return OUT
 
 
