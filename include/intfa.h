@@ -121,9 +121,10 @@ typedef struct intfa_fwd_params {
     int64_t vs_stride_blk;    /* elements between consecutive scale rows of v_scale (>= head_dim) */
     const int32_t* seqlens_k; /* optional device array [batch]: number of keys of each batch entry, 0 <= n <= seqlen_k (a
                                  key/value cache filled to different lengths; the counterpart of the reference's
-                                 cu_seqlens_k used as lengths / seqused_k, csrc/flash.h:95-99,149-151, csrc/block_info.h:21-22).  k, v and k_scale keep their seqlen_k-row
-                                 layout; rows past a batch entry's length are not read.  An entry with no key gives zeros
-                                 (lse = -inf).  NULL = every entry has seqlen_k keys.  Not with causal. */
+                                 seqused_k and of cu_seqlens_k used as lengths, csrc/flash.h:95-99,149-151,
+                                 csrc/block_info.h:21-22).  k, v and k_scale keep their seqlen_k-row layout; rows past a
+                                 batch entry's length are not read.  An entry with no key gives zeros (lse = -inf).
+                                 NULL = every entry has seqlen_k keys.  Not with causal. */
 } intfa_fwd_params;
 
 /* Library/ABI version (INTFA_VERSION of the build). */
@@ -134,7 +135,9 @@ const char* intfa_error_string(int code);
 
 /* Key-block length of a variant at a head_dim (the reference's BLOCK_N, an autotuned value there:
  * configs.py:13-19).  The running max and, on the full-int8 path, the requantisation of P advance per key block,
- * so a bit-faithful CPU evaluation must use the same value.  Negative INTFA_ERR_* for unknown arguments. */
+ * so a bit-faithful CPU evaluation must use the same value.  It holds for every shape: the kernel that takes over
+ * decode-shaped calls (at most 64 query rows, no causal mask, head_dim <= 128) walks the same blocks.
+ * Negative INTFA_ERR_* for unknown arguments. */
 int intfa_fwd_block_n(int variant, int head_dim);
 
 /* A split count for the problem in *p (its num_splits and workspace members are ignored): 1 when the single-pass grid
