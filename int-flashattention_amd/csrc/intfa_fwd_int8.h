@@ -420,9 +420,19 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
 #pragma unroll
                 for (int b4 = 0; b4 < 4; ++b4) {
                     const int r = 4 * a4 + b4;
-                    if (VBLK) o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, (float)oacc[dt & 1][r] * vsc[dt & 1][a4][b4]);
-                    else o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, (float)oacc[dt & 1][r]);
-                    asm volatile("" : "+v"(o_acc[dt][r]));     // keeps the update in this slot (it would be sunk below the loop)
+                    float pv = (float)oacc[dt & 1][r];
+                    if (VBLK) pv *= vsc[dt & 1][a4][b4];
+                    // o = o * alpha + pv, written as the three-operand instruction in place: left to the compiler the
+                    // update is either sunk below the loop (no vector work beside the MFMAs of this stage) or, pinned
+                    // here by an empty asm, emitted as v_fmac into the temporary plus a copy back (one instruction more
+                    // per output element and block).  At head_dim 256 the register allocation is tighter and the
+                    // pinned form, which leaves the choice of registers to the compiler, does not spill.
+                    if (D <= 128) {
+                        asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(o_acc[dt][r]) : "v"(alpha), "v"(pv));
+                    } else {
+                        o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, pv);
+                        asm volatile("" : "+v"(o_acc[dt][r]));
+                    }
                 }
             }
         }
