@@ -342,6 +342,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         // -------- pass 2: P = exp2(x*qsc - m), row sum, requantise
         float lsum = 0.f;
         v4i p8[NST];
+        v16i oacc[2];
         const float bias = (PROUND == 0 ? kLog2_127 : 0.f) - m_new;
 #pragma unroll
         for (int st = 0; st < NST; ++st) {
@@ -376,10 +377,15 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                 p8[st][w4] = (int)pk;
             }
             asm volatile("" : "+v"(lsum));      // keep the row-sum chain inside its stage
+            // the P V chain of the first d-tile advances by one MFMA as soon as this sub-tile's P8 is packed: it runs
+            // under the exponentials of the next sub-tile instead of in a burst behind the pass
+            if (!(DIAG && st > gw)) {
+                if (st == 0) oacc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][0], p8[0], (v16i){0}, 0, 0, 0);
+                else oacc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][st], p8[st], oacc[0], 0, 0, 0);
+            }
         }
         // -------- P V on int8 MFMA: O^T[d, q] += V^T[d, key] P^T[key, q]; the chain of d-tile dt+1 is issued
         // before the accumulator update of d-tile dt, its V fragments were requested two stages earlier.
-        v16i oacc[2];
         constexpr int VSB = BUF * DV * 4;
         v4f vsc[2][4];                          // VBLK: channel scales of the d-tile being folded in / the next one
         auto load_vsc = [&](v4f (&dst)[4], int dt) __attribute__((always_inline)) {
@@ -387,16 +393,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             for (int a4 = 0; a4 < 4; ++a4) dst[a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (32 * dt + 8 * a4));
         };
         if (VBLK) load_vsc(vsc[0], 0);
-        auto pv_chain = [&](v16i& acc, const v4i (&f)[NST]) __attribute__((always_inline)) {
-            acc = (v16i){0};
-#pragma unroll
-            for (int st = 0; st < NST; ++st) {
-                if (DIAG && st > gw) continue;
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[st], p8[st], acc, 0, 0, 0);
-            }
-        };
         __builtin_amdgcn_sched_barrier(0);
-        pv_chain(oacc[0], vf[0]);
         // As in pass 1: the MFMAs of d-tile dt+1 are issued one at a time between quarters of the accumulator update
         // of d-tile dt.
 #pragma unroll
