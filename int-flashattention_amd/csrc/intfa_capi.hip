@@ -3,7 +3,6 @@
 #include "intfa_device.h"
 #include "intfa_launch.h"
 #include "intfa_splitkv.h"
-#include "intfa_fwd_decode.h"
 
 using namespace intfa;
 
@@ -12,8 +11,6 @@ namespace {
 constexpr int kMaxSplits = 64;
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
-int scale_size(int dt) { return dt == INTFA_F32 ? 4 : 2; }
 
 // Key-block length of a variant at a head_dim: the full-int8 kernel takes 128 keys per block (64 at head_dim 256),
 // the kernels with a 16-bit P V take 64.

@@ -15,10 +15,9 @@
 // start of a block (the data comes from HBM, not from a cache shared with other query blocks).
 #pragma once
 #include "intfa_device.h"
+#include "intfa_launch.h"
 
 namespace intfa {
-
-constexpr int kDecodeRows = 32;       // query rows per workgroup of the decode kernel
 
 // Head dims 64 and 128 (the key block of the general kernel is 128 there too, so both kernels evaluate the same blocks).
 template <int D, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool SPLIT, bool VBLK>

@@ -5,6 +5,8 @@
 
 namespace intfa {
 
+constexpr int kDecodeRows = 32;       // query rows per workgroup of the decode-shaped kernel (intfa_fwd_decode.h)
+
 // Launch switches resolved to template arguments inside the instance files.
 struct LaunchSel {
     bool causal;
