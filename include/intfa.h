@@ -49,7 +49,7 @@ enum {
     INTFA_OK = 0,
     INTFA_ERR_NULL = -1,          /* a required pointer is NULL */
     INTFA_ERR_HEAD_DIM = -2,      /* head_dim not supported by the kernels */
-    INTFA_ERR_SEQLEN = -3,        /* seqlen not positive, or causal with seqlen_k != seqlen or with seqlens_k */
+    INTFA_ERR_SEQLEN = -3,        /* seqlen not positive or seqlen_k negative */
     INTFA_ERR_ALIGN = -4,         /* pointer or row stride not 16-byte aligned */
     INTFA_ERR_DTYPE = -5,         /* unknown dtype enum */
     INTFA_ERR_WORKSPACE = -6,     /* workspace missing or too small for the requested split count */
@@ -92,7 +92,10 @@ typedef struct intfa_fwd_params {
     int32_t batch, heads, seqlen, head_dim;
     int32_t scale_dtype;      /* INTFA_F16 / INTFA_BF16 / INTFA_F32 */
     int32_t io_dtype;         /* type of out (and of fp q/k/v): INTFA_F16 or INTFA_BF16 */
-    int32_t causal;           /* 0 / 1; queries and keys share positions (seqlen_q == seqlen_k) */
+    int32_t causal;           /* 0 / 1.  Query row i sees keys 0 .. i + (seqlen_k - seqlen): with equal lengths the reference's
+                                 mask (flash_atten_full_int8.py:39-43); with more keys than queries (a chunk of new tokens
+                                 against a cache) the mask is aligned to the bottom right corner as in the reference's CUDA
+                                 tree (csrc/mask.h:53,172).  A row that sees no key (fewer keys than queries) gives zeros. */
     float   sm_scale;
     int32_t p_round;          /* INTFA_PROUND_* (full-int8 only) */
 
@@ -107,8 +110,7 @@ typedef struct intfa_fwd_params {
                                  0 or heads = one K/V head per query head (the reference's Python API; its CUDA tree
                                  has the grouped form, csrc/flash_fwd_kernel_full_qi8.h:141).  Must divide heads. */
     int32_t seqlen_k;         /* number of keys when it differs from the number of queries (cross attention, decoding
-                                 against a cache): k, v and k_scale then have seqlen_k rows.  0 = seqlen.  Not with
-                                 causal (the reference's mask is defined for equal lengths). */
+                                 against a cache): k, v and k_scale then have seqlen_k rows.  0 = seqlen. */
     int32_t v_scale_block;    /* full-int8 only.  0: one V scale per (batch, head), the reference's Python API
                                  (flash_atten_full_int8.py:159-161).  > 0: V was quantised per block of v_scale_block keys
                                  and per channel, the layout its CUDA kernel reads (csrc/flash_fwd_kernel_full_qi8.h:
@@ -124,7 +126,8 @@ typedef struct intfa_fwd_params {
                                  seqused_k and of cu_seqlens_k used as lengths, csrc/flash.h:95-99,149-151,
                                  csrc/block_info.h:21-22).  k, v and k_scale keep their seqlen_k-row layout; rows past a
                                  batch entry's length are not read.  An entry with no key gives zeros (lse = -inf).
-                                 NULL = every entry has seqlen_k keys.  Not with causal. */
+                                 NULL = every entry has seqlen_k keys.  With causal the mask of an entry is aligned to
+                                 its own length. */
 } intfa_fwd_params;
 
 /* Library/ABI version (INTFA_VERSION of the build). */

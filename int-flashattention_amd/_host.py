@@ -65,8 +65,6 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
     N_k = k.shape[2]
     if k.shape[0] != Z or v.shape[0] != Z or v.shape[2] != N_k or v.shape[1] != H_kv:
         raise ValueError("q, k and v must share the batch size, and k and v their heads and length")
-    if causal and N_k != N:
-        raise ValueError("causal attention needs as many keys as queries (the reference passes a single N_CTX)")
     if H % H_kv != 0:
         raise ValueError(f"the number of query heads ({H}) must be a multiple of the number of K/V heads ({H_kv})")
     dk = max(d, MIN_HEAD_DIM)
@@ -117,8 +115,6 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
     if seqlens_k is not None:
         # number of keys per batch entry (a cache filled to different lengths); int32 [Z] on the device
         _require_gpu(seqlens_k)
-        if causal:
-            raise ValueError("per-batch key lengths are for non-causal attention (decoding against a cache)")
         if seqlens_k.dtype != torch.int32 or tuple(seqlens_k.shape) != (Z,):
             raise ValueError(f"seqlens_k must be an int32 tensor of shape ({Z},)")
         seqlens_k = seqlens_k.contiguous()

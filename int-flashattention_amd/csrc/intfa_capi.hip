@@ -27,7 +27,6 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
     if (heads_kv > p->heads || p->heads % heads_kv != 0) return INTFA_ERR_SHAPE;
     if (p->seqlen <= 0 || p->seqlen_k < 0) return INTFA_ERR_SEQLEN;
     const int seqlen_k = p->seqlen_k > 0 ? p->seqlen_k : p->seqlen;
-    if (p->causal && seqlen_k != p->seqlen) return INTFA_ERR_SEQLEN;      // the causal mask is defined for equal lengths
     if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256) return INTFA_ERR_HEAD_DIM;
     if (p->scale_dtype < 0 || p->scale_dtype > 2) return INTFA_ERR_DTYPE;
     if (p->io_dtype != INTFA_F16 && p->io_dtype != INTFA_BF16) return INTFA_ERR_DTYPE;
@@ -75,7 +74,6 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
     }
     k.lse = p->lse;
     if (p->seqlens_k != nullptr) {
-        if (p->causal) return INTFA_ERR_SEQLEN;                              // as seqlen_k: no causal mask over two lengths
         if (reinterpret_cast<uintptr_t>(p->seqlens_k) & 3u) return INTFA_ERR_ALIGN;
         k.seqlens_k = p->seqlens_k;
     }
@@ -192,7 +190,7 @@ const char* intfa_error_string(int code) {
         case INTFA_OK: return "ok";
         case INTFA_ERR_NULL: return "a required pointer is NULL";
         case INTFA_ERR_HEAD_DIM: return "head_dim must be 64, 128 or 256";
-        case INTFA_ERR_SEQLEN: return "seqlen must be positive; seqlen_k, when set, must equal it for causal attention";
+        case INTFA_ERR_SEQLEN: return "seqlen must be positive and seqlen_k not negative";
         case INTFA_ERR_ALIGN: return "pointers and row/head/batch strides must be 16-byte aligned";
         case INTFA_ERR_DTYPE: return "unknown dtype enum";
         case INTFA_ERR_WORKSPACE: return "workspace missing, misaligned or too small for num_splits";

@@ -33,7 +33,6 @@ template <bool QK_INT8, int D, bool CAUSAL, int IO_DT, bool SPLIT>
 __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr int BN = kBlockN16, NST = BN / 32;
-    constexpr int RDIAG = kBlockM / BN;               // key blocks overlapping the diagonal of a query block
     constexpr int QB = QK_INT8 ? 1 : 2;               // bytes per Q/K element
     constexpr int KROW = D * QB, VROW = D * 2;        // bytes per K / V row
     constexpr int KS = KROW / 32;                     // MFMA k-steps of S^T (32 bytes of a row each)
@@ -98,7 +97,13 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
         seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
     }
     const int nb_total = (seqlen_k + BN - 1) / BN;
-    int nb_begin = 0, nb_end = CAUSAL ? ((mb + 1) * RDIAG < nb_total ? (mb + 1) * RDIAG : nb_total) : nb_total;
+    // causal mask aligned to the bottom right corner as in the full-int8 kernel: row i sees keys 0 .. i + causal_off
+    const int causal_off = seqlen_k - p.seqlen;
+    int nb_begin = 0, nb_end = nb_total;
+    if (CAUSAL) {
+        const int e = (mb * kBlockM + kBlockM + causal_off + BN - 1) / BN;
+        nb_end = e < 0 ? 0 : (e < nb_total ? e : nb_total);
+    }
     if (SPLIT) {
         // non-causal: the key blocks of the sequence are dealt evenly to the splits (csrc/flash_fwd_kernel.h:503-511);
         // causal: the blocks VISIBLE to this query block are, so that no split of a query block is empty or short
@@ -187,10 +192,10 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     // barriers: the MFMAs of S^T sub-tile st+1 are issued one at a time between quarters of the vector work of sub-tile
     // st, the MFMAs of output d-tile dt between quarters of the rescaling of d-tile dt+1, and LDS operands are requested
     // one or two stages before the MFMA that consumes them.
-    // DIAG selects the code instance with masking: sub-tiles st > gw are skipped, in sub-tile gw the keys whose index
-    // inside the sub-tile exceeds `lim` are masked (causal diagonal: gw = the wave's own sub-tile, lim = the lane's
-    // row; ragged last block: the position of the last valid key).
-    auto compute = [&](auto buf_tag, auto diag_tag, int nb, int gw, int lim) __attribute__((always_inline)) {
+    // DIAG selects the code instance with masking: keys whose index inside the block exceeds the lane's `lim` are masked
+    // and sub-tiles st > gw (wave-uniform: the sub-tile of the largest lim in the wave) are skipped (causal diagonal:
+    // lim = the lane's last visible key; ragged last block: the last valid key).
+    auto compute = [&](auto buf_tag, auto diag_tag, int nb, int gw, int lim, int lim_lo) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         constexpr bool DIAG = decltype(diag_tag)::value;
         constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4;
@@ -255,7 +260,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
                 for (int b4 = 0; b4 < 4; ++b4) {
                     const int r = 4 * a4 + b4;
                     float v = QK_INT8 ? (float)si[st][r] * kk[st][a4][b4] : sf[st][r];
-                    if (DIAG && st == gw && (8 * a4 + b4 + 4 * lh) > lim) v = -INFINITY;
+                    if (DIAG && 32 * st + 31 > lim_lo && (32 * st + 8 * a4 + b4 + 4 * lh) > lim) v = -INFINITY;
                     t[st][r] = v;
                     mx = fmaxf(mx, v);
                 }
@@ -312,14 +317,14 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
         }
     };
 
-    auto step = [&](auto buf_tag, auto diag_tag, int nb, int gw, int lim) __attribute__((always_inline)) {
+    auto step = [&](auto buf_tag, auto diag_tag, int nb, int gw, int lim, int lim_lo) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         const bool more = nb + 1 < nb_end;
         uint32_t ks_next = 0;
         if (more) { issue_loads(nb + 1, BUF ^ 1); ks_next = load_ks(nb + 1); }
-        compute(buf_tag, diag_tag, nb, gw, lim);
+        compute(buf_tag, diag_tag, nb, gw, lim, lim_lo);
         if (QK_INT8 && more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
     };
 
@@ -329,26 +334,27 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
             const uint32_t s0 = load_ks(nb_begin);
             if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
         }
-        const int diag_begin = mb * RDIAG;
+        const int diag_first = (mb * kBlockM + causal_off + 1) / BN;   // first block with a key hidden from the block's first row
+        const int diag_begin = diag_first < 0 ? 0 : diag_first;
         const int tail_keys = seqlen_k - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
         const bool ragged = !CAUSAL && tail_keys < BN && nb_end == nb_total;
         const int plain_end = CAUSAL ? (nb_end > diag_begin ? diag_begin : nb_end) : (ragged ? nb_end - 1 : nb_end);
         int nb = nb_begin;
         while (true) {
             if (nb >= plain_end) break;
-            step(BoolTag<false>{}, BoolTag<false>{}, nb++, 0, 0);
+            step(BoolTag<false>{}, BoolTag<false>{}, nb++, 0, 0, 0);
             if (nb >= plain_end) break;
-            step(BoolTag<true>{}, BoolTag<false>{}, nb++, 0, 0);
+            step(BoolTag<true>{}, BoolTag<false>{}, nb++, 0, 0, 0);
         }
-        // masked blocks: the blocks on the causal diagonal, or the ragged last block of a non-causal pass
-#pragma unroll
-        for (int kb = 0; kb < (CAUSAL ? RDIAG : 1); ++kb) {
-            if (nb >= nb_end) break;
-            const int gw = CAUSAL ? wave - (nb - diag_begin) * NST : (tail_keys - 1) >> 5;
-            const int lim = CAUSAL ? lq : (tail_keys - 1) & 31;
-            if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb, gw, lim);
-            else step(BoolTag<true>{}, BoolTag<true>{}, nb, gw, lim);
-            ++nb;
+        // masked blocks: the blocks the causal diagonal of this query block crosses, or the ragged last block of a
+        // non-causal pass
+#pragma clang loop unroll(disable)
+        for (; nb < nb_end; ++nb) {
+            const int lim = CAUSAL ? q_row + causal_off - nb * BN : tail_keys - 1;
+            const int gw = (CAUSAL ? mb * kBlockM + wave * 32 + 31 + causal_off - nb * BN : tail_keys - 1) >> 5;
+            const int lim_lo = CAUSAL ? mb * kBlockM + wave * 32 + causal_off - nb * BN : tail_keys - 1;   // smallest lim in the wave
+            if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb, gw, lim, lim_lo);
+            else step(BoolTag<true>{}, BoolTag<true>{}, nb, gw, lim, lim_lo);
         }
     }
 
@@ -359,7 +365,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     const int eb = head / e_heads, eh = head % e_heads;
     const float l_tot = half_pair_sum(l_run);
     // (no key at all - an empty cache entry - gives zeros and lse = -inf instead of 0 / 0)
-    const bool any_key = nb_begin < nb_end;
+    const bool any_key = nb_begin < nb_end && m_run > -INFINITY;      // (a causal row above the first key sees nothing)
     const float inv = any_key ? 1.f / l_tot : 0.f;
     const float lse = any_key ? m_run + __builtin_log2f(l_tot) : -INFINITY;
     if (SPLIT) {
@@ -392,12 +398,12 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
             if (IO_DT == 0) {
                 v4h o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(o_acc[dt][4 * a4 + b4] * inv);
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(any_key ? o_acc[dt][4 * a4 + b4] * inv : 0.f);
                 *(v4h*)(orow + d0 * 2) = o;
             } else {
                 v4s o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(o_acc[dt][4 * a4 + b4] * inv);
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(any_key ? o_acc[dt][4 * a4 + b4] * inv : 0.f);
                 *(v4s*)(orow + d0 * 2) = o;
             }
         }

@@ -39,7 +39,6 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     constexpr int DT = DV / 32;                  // 32-wide output tiles along head_dim
     constexpr int NST = FullInt8Geom<D>::NST;    // 32-key sub-tiles per key block
     constexpr int BN = FullInt8Geom<D>::BN;      // keys per block
-    constexpr int RDIAG = kBlockM / BN;          // key blocks that overlap the causal diagonal of a query block
     constexpr int KT = BN * D;                   // bytes of one K tile
     constexpr int VT = BN * DV;                  // bytes of one int8 V tile (this workgroup's columns)
     constexpr int CH = D / 16;                   // 16-byte chunks per K row
@@ -111,7 +110,14 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
     }
     const int nb_total = (seqlen_k + BN - 1) / BN;
-    int nb_begin = 0, nb_end = CAUSAL ? ((mb + 1) * RDIAG < nb_total ? (mb + 1) * RDIAG : nb_total) : nb_total;
+    // Causal mask aligned to the bottom right corner (csrc/mask.h:53,172 of the reference's CUDA tree): query row i sees
+    // keys 0 .. i + causal_off.  Equal lengths (the reference's Python API) give causal_off = 0.
+    const int causal_off = seqlen_k - p.seqlen;
+    int nb_begin = 0, nb_end = nb_total;
+    if (CAUSAL) {                                          // blocks that hold a key visible to the last row of this query block
+        const int e = (mb * kBlockM + kBlockM + causal_off + BN - 1) / BN;
+        nb_end = e < 0 ? 0 : (e < nb_total ? e : nb_total);
+    }
     if (SPLIT) {
         // non-causal: the key blocks of the sequence are dealt evenly to the splits (csrc/flash_fwd_kernel.h:503-511);
         // causal: the blocks VISIBLE to this query block are, so that no split of a query block is empty or short
@@ -227,10 +233,10 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     const uint32_t ks_wr = OFF_KS + 4 * (tid & (BN - 1));
 
     // One key block out of LDS buffer BUF.  DIAG selects the code for the block on the causal diagonal.
-    // DIAG selects the code instance with masking: sub-tiles st > gw of the block are skipped, in sub-tile gw the keys
-    // whose index inside the sub-tile exceeds `lim` are masked.  Causal diagonal: gw = the wave's own sub-tile,
-    // lim = the lane's row (key <= query); last block of a ragged sequence: gw, lim = position of the last valid key.
-    auto compute = [&](auto buf_tag, auto diag_tag, int nb, bool more, int gw_in, int lim) __attribute__((always_inline)) {
+    // DIAG selects the code instance with masking: keys whose index inside the block exceeds the lane's `lim` are masked
+    // and sub-tiles st > gw (wave-uniform, the sub-tile of the largest lim in the wave) are skipped.  Causal diagonal:
+    // lim = the lane's last visible key; last block of a ragged sequence: lim = the last valid key.
+    auto compute = [&](auto buf_tag, auto diag_tag, int nb, bool more, int gw_in, int lim, int lim_lo) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         constexpr bool DIAG = decltype(diag_tag)::value;
         constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4;
@@ -317,13 +323,17 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
+                float xq[4];
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) xq[b4] = (float)acc[4 * a4 + b4] * kk[st & 1][a4][b4];
+                if (DIAG && 32 * st + 31 > lim_lo) {           // wave-uniform: some lane of the wave has a hidden key in this sub-tile
+#pragma unroll
+                    for (int b4 = 0; b4 < 4; ++b4)
+                        if ((32 * st + 8 * a4 + b4 + 4 * lh) > lim) xq[b4] = -INFINITY;
+                }
 #pragma unroll
                 for (int b4 = 0; b4 < 4; ++b4) {
-                    float x = (float)acc[4 * a4 + b4] * kk[st & 1][a4][b4];
-                    if (DIAG) {
-                        // position of the key inside the 32x32 tile on the diagonal vs this lane's query
-                        if (st == gw && (8 * a4 + b4 + 4 * lh) > lim) x = -INFINITY;
-                    }
+                    const float x = xq[b4];
                     t[st][4 * a4 + b4] = x;
                     mx = fmaxf(mx, x);
                 }
@@ -438,7 +448,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
 
     // One pipeline step on LDS buffer BUF: wait for this block's tiles (issued one step earlier), make them
     // visible to all four waves, start the copy of the next block into the other buffer, compute.
-    auto step = [&](auto buf_tag, auto diag_tag, int nb, int gw, int lim) __attribute__((always_inline)) {
+    auto step = [&](auto buf_tag, auto diag_tag, int nb, int gw, int lim, int lim_lo) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -451,7 +461,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             ks_next = load_ks(nb + 1);
             if (vs_thread) vs_next = load_vs(nb + 1);
         }
-        compute(buf_tag, diag_tag, nb, more, gw, lim);
+        compute(buf_tag, diag_tag, nb, more, gw, lim, lim_lo);
         if (more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
         if (more && vs_thread) *(float*)(smem + vs_wr + (BUF ^ 1) * DV * 4) = vs_next;
     };
@@ -465,27 +475,32 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
             if (vs_thread) *(float*)(smem + vs_wr) = load_vs(nb_begin);
         }
-        const int diag_begin = mb * RDIAG;                 // first key block that touches the diagonal
+        // first key block that holds a key hidden from the first row of this query block (every block before it is
+        // visible to all rows and runs without a mask)
+        const int diag_first = (mb * kBlockM + causal_off + 1) / BN;
+        const int diag_begin = diag_first < 0 ? 0 : diag_first;
         const int tail_keys = seqlen_k - (nb_total - 1) * BN;        // valid keys of the last block (BN if it is full)
         const bool ragged = !CAUSAL && tail_keys < BN && nb_end == nb_total;
         const int plain_end = CAUSAL ? (nb_end > diag_begin ? diag_begin : nb_end) : (ragged ? nb_end - 1 : nb_end);
         int nb = nb_begin;
         while (true) {
             if (nb >= plain_end) break;
-            step(BoolTag<false>{}, BoolTag<false>{}, nb++, 0, 0);
+            step(BoolTag<false>{}, BoolTag<false>{}, nb++, 0, 0, 0);
             if (nb >= plain_end) break;
-            step(BoolTag<true>{}, BoolTag<false>{}, nb++, 0, 0);
+            step(BoolTag<true>{}, BoolTag<false>{}, nb++, 0, 0, 0);
         }
-        // masked blocks: up to RDIAG blocks on the causal diagonal (keys past the end of a ragged sequence lie above
+        // masked blocks: the blocks the causal diagonal of this query block crosses (kBlockM / BN of them when the lengths
+        // are equal, one more when the offset is not a multiple of the block; keys past the end of a ragged sequence lie above
         // every valid row's diagonal), or the ragged last block of a non-causal pass
-#pragma unroll
-        for (int kb = 0; kb < (CAUSAL ? RDIAG : 1); ++kb) {
-            if (nb >= nb_end) break;
-            const int gw = CAUSAL ? wave - (nb - diag_begin) * NST : (tail_keys - 1) >> 5;
-            const int lim = CAUSAL ? lq : (tail_keys - 1) & 31;
-            if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb, gw, lim);
-            else step(BoolTag<true>{}, BoolTag<true>{}, nb, gw, lim);
-            ++nb;
+#pragma clang loop unroll(disable)
+        for (; nb < nb_end; ++nb) {
+            // lane: last visible key relative to the block; wave: sub-tile of the largest of them (negative: none)
+            const int lim = CAUSAL ? q_row + causal_off - nb * BN : tail_keys - 1;
+            const int gw = (CAUSAL ? mb * kBlockM + wave * 32 + 31 + causal_off - nb * BN : tail_keys - 1) >> 5;
+            // smallest lim in the wave: sub-tiles that end at or below it need no per-key test
+            const int lim_lo = CAUSAL ? mb * kBlockM + wave * 32 + causal_off - nb * BN : tail_keys - 1;
+            if (((nb - nb_begin) & 1) == 0) step(BoolTag<false>{}, BoolTag<true>{}, nb, gw, lim, lim_lo);
+            else step(BoolTag<true>{}, BoolTag<true>{}, nb, gw, lim, lim_lo);
         }
     }
     if (DUMP_S) return;
@@ -498,8 +513,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     const int eb = head / e_heads, eh = head % e_heads;
     const float l_tot = half_pair_sum(l_run);          // in units of 1/127 when PROUND == 0
     const float vs = VBLK ? 1.f : load_scale(pe->v_scale, eb * pe->vs_sb + (eh / pe->kv_group) * pe->vs_sh, pe->scale_dtype);
-    // (no key at all - an empty cache entry - gives zeros and lse = -inf instead of 0 / 0)
-    const bool any_key = nb_begin < nb_end;
+    // (no visible key at all - an empty cache entry, or a causal row above the first key when there are fewer keys than
+    // queries - gives zeros and lse = -inf; such a row's accumulators hold NaN from exp2(-inf - -inf), hence the selects)
+    const bool any_key = nb_begin < nb_end && m_run > -INFINITY;
     const float out_scale = !any_key ? 0.f : (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
     const float l_true = (PROUND == 0) ? l_tot * (1.f / 127.f) : l_tot;
     const float lse = any_key ? m_run + __builtin_log2f(l_true) : -INFINITY;
@@ -533,12 +549,12 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             if (OUT_DT == 0) {
                 v4h o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(o_acc[dt][4 * a4 + b4] * out_scale);
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(any_key ? o_acc[dt][4 * a4 + b4] * out_scale : 0.f);
                 *(v4h*)(orow + d0 * 2) = o;
             } else {
                 v4s o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(o_acc[dt][4 * a4 + b4] * out_scale);
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(any_key ? o_acc[dt][4 * a4 + b4] * out_scale : 0.f);
                 *(v4s*)(orow + d0 * 2) = o;
             }
         }

@@ -20,8 +20,10 @@ def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, *,
     ``quant_perblock_channel``.  ``v_scale_block`` defaults to the kernel's key-block length (``block_n("full", d)``)
     and must be a multiple of it.
 
-    ``seqlens_k`` (int32 [Z] on the device, non-causal only): number of keys of each batch entry when k and v are a cache
-    filled to different lengths; rows past an entry's length are not read.
+    k and v may have another length than q (and fewer heads: grouped-query attention).  With ``causal`` query row i then
+    sees keys 0 .. i + Nk - Nq (mask aligned to the bottom right corner: new tokens against a cache).
+    ``seqlens_k`` (int32 [Z] on the device): number of keys of each batch entry when k and v are a cache filled to
+    different lengths; rows past an entry's length are not read.
 
     ``p_round``: "rne" folds 127 into the exponent and rounds to nearest-even; "reference" reproduces the
     fp16 sequence of flash_atten_full_int8.py:49-51.

@@ -41,8 +41,10 @@ How every function is pinned (tests/test_oracle.py):
   is that constant times sum(P8)/(127 l).
 * causal: equality with a dense tril-masked evaluation; first row attends to key 0 only.
 * split-KV: any split count agrees with one split to fp32 rounding.
-* separate query and key lengths (non-causal): rows are independent, so a slice of the query rows against the full keys
-  must reproduce the same rows of the square evaluation bit for bit.
+* separate query and key lengths: rows are independent, so a slice of the query rows against the full keys must
+  reproduce the same rows of the square evaluation bit for bit; causal with the mask aligned to the bottom right corner:
+  the last Nq rows of the square causal problem, bit for bit; with fewer keys than queries the first rows see nothing
+  and give zeros.
 * blocked V scales: a 4-D scale tensor filled with one value per (batch, head) reproduces the scalar form bit for
   bit; the result equals the scalar form applied to V pre-multiplied by the block/channel factors when these are
   powers of two; ``quant_perblock_channel`` against a pure-Python loop, and every (block, channel) reaches +-127.
@@ -117,8 +119,8 @@ def attention_exact(q, k, v, causal: bool, sm_scale: float) -> torch.Tensor:
     qf, kf, vf = q.float(), k.float(), v.float()
     p = torch.matmul(qf, kf.transpose(2, 3)) * sm_scale
     if causal:
-        n = q.shape[2]
-        mask = torch.tril(torch.ones((n, n), dtype=torch.bool))
+        n, nk = q.shape[2], k.shape[2]           # equal in the reference; otherwise the mask is aligned bottom right
+        mask = (torch.arange(n)[:, None] + (nk - n)) >= torch.arange(nk)[None, :]
         p = p.masked_fill(~mask, float("-inf"))
     p = torch.softmax(p, dim=-1).to(q.dtype if q.dtype.is_floating_point else torch.float16).float()
     return torch.matmul(p, vf).to(q.dtype if q.dtype.is_floating_point else torch.float16)
@@ -178,8 +180,11 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
     (csrc/mask.h:313-340); ``v_scale_block`` must be a multiple of ``block_n``.
     """
     B, H, N, D = q.shape
-    Nk = k.shape[2]                # differs from N for cross attention / decoding against a cache (non-causal only)
-    assert not causal or Nk == N   # the reference's mask is defined for one N_CTX (flash_atten_full_int8.py:213)
+    Nk = k.shape[2]                # differs from N for cross attention / a chunk of new tokens against a cache
+    # causal: row i sees keys 0 .. i + off.  off = 0 is the reference's Python API (one N_CTX, flash_atten_full_int8.py:213);
+    # with more keys than queries the mask is aligned to the bottom right corner as in its CUDA tree (csrc/mask.h:53,172:
+    # col_idx_limit_right = row_idx + 1 + max_seqlen_k - max_seqlen_q)
+    off = Nk - N
     key_hi = Nk if key_hi is None else key_hi
     row_hi = N if row_hi is None else row_hi
     # N need not be a multiple of the blocks: the last key block and the last row tile are simply shorter, which is
@@ -206,9 +211,16 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
     for start_n in range(key_lo, key_hi, block_n):
         kj = k[:, :, start_n:start_n + block_n]
         vj = v[:, :, start_n:start_n + block_n]
-        if causal:
+        if causal and off == 0:
             tile = start_n // block_m
             segments = [(tile * block_m, min((tile + 1) * block_m, N), True), ((tile + 1) * block_m, N, False)]
+        elif causal:
+            # rows that see a part of this block (masked evaluation) and rows that see all of it; rows above see nothing.
+            # (For rows that see the whole block the two evaluations give identical numbers, so where the boundary
+            # between the segments lies does not matter.)
+            end_n = min(start_n + block_n, key_hi)
+            lo, hi = min(max(start_n - off, 0), N), min(max(end_n - off, 0), N)
+            segments = [(lo, hi, True), (hi, N, False)]
         else:
             segments = [(0, N, False)]
         for r0, r1, masked in segments:
@@ -224,7 +236,7 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
                 qk = torch.matmul(qi.float(), kj.float().transpose(2, 3))    # flash_atten_fp.py:33
             m_i = m[:, :, r0:r1]
             if masked:                                                       # :39-43
-                keep = rows[r0:r1, None] >= (start_n + torch.arange(kj.shape[2]))[None, :]
+                keep = (rows[r0:r1, None] + off) >= (start_n + torch.arange(kj.shape[2]))[None, :]
                 qk = qk * qk_scale + torch.where(keep, 0.0, -1.0e6)
                 m_ij = torch.maximum(m_i, qk.max(dim=-1).values)
                 qk = qk - m_ij[..., None]
@@ -329,6 +341,7 @@ def attention_full_int8_splitkv(q, k, v, q_scale, k_scale, v_scale, causal: bool
     """Full-int8 forward evaluated as ``num_splits`` independent key ranges merged by ``splitkv_combine``: the ranges of
     ``splitkv_ranges`` for a non-causal pass, those of ``splitkv_ranges_causal`` (per row tile) for a causal one."""
     B, H, N, D = q.shape
+    assert not causal or k.shape[2] == N      # the causal partition below is the one of equal lengths
     o_parts = torch.zeros((num_splits, B, H, N, D))
     lse_parts = torch.full((num_splits, B, H, N), float("-inf"))
     if causal:

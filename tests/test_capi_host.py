@@ -68,7 +68,6 @@ def _valid_block():
     (lambda p: setattr(p, "v_scale", None), -1),
     (lambda p: setattr(p, "head_dim", 48), -2),
     (lambda p: setattr(p, "seqlen", -128), -3),
-    (lambda p: (setattr(p, "causal", 1), setattr(p, "seqlen_k", 512)), -3),    # causal with a different key length
     (lambda p: setattr(p, "seqlen", 0), -3),
     (lambda p: setattr(p, "k", 0x10008), -4),
     (lambda p: setattr(p, "q_stride_n", 120), -4),
@@ -83,7 +82,7 @@ def _valid_block():
     (lambda p: (setattr(p, "v_scale_block", 64), setattr(p, "vs_stride_blk", 128)), -9),    # not a multiple of the key block (128)
     (lambda p: (setattr(p, "v_scale_block", 128), setattr(p, "vs_stride_blk", 64)), -9),    # scale rows overlap
     (lambda p: setattr(p, "v_scale_block", -1), -9),
-    (lambda p: (setattr(p, "causal", 1), setattr(p, "seqlens_k", 0x10000)), -3),        # per-batch key lengths are non-causal
+    (lambda p: setattr(p, "seqlen_k", -5), -3),
     (lambda p: setattr(p, "seqlens_k", 0x10002), -4),
     (lambda p: (setattr(p, "v_scale_block", 128), setattr(p, "vs_stride_blk", 128), setattr(p, "v_scale", 0x10002)), -4),
 ])

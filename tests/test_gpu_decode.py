@@ -178,7 +178,3 @@ def test_per_batch_key_lengths_with_split_kv_and_argument_checks():
         M.attention_full_int8(*args, False, sm, seqlens_k=sl.long())
     with pytest.raises(ValueError):
         M.attention_full_int8(*args, False, sm, seqlens_k=sl[:2])
-    sq = decode_inputs(1, 2, 2, 128, 128, 64, seed=97)
-    with pytest.raises(ValueError):
-        M.attention_full_int8(*gpu(sq["q8"], sq["k8"], sq["v8"], sq["qs"], sq["ks"], sq["vs"]), True, 0.1,
-                              seqlens_k=torch.tensor([128], dtype=torch.int32, device=DEV))

@@ -443,11 +443,68 @@ def test_grouped_decoding_folds_heads_into_rows(Nq):
     assert torch.equal(o, o_rep)
 
 
-def test_causal_needs_equal_lengths():
-    q = torch.zeros((1, 1, 128, 64), dtype=torch.float16, device=DEV)
-    k = torch.zeros((1, 1, 256, 64), dtype=torch.float16, device=DEV)
-    with pytest.raises(ValueError, match="causal"):
-        M.attention(q, k, k, True, 1.0)
+@pytest.mark.parametrize("variant", ["full", "half", "fp"])
+@pytest.mark.parametrize("Nq,Nk,D", [(128, 256, 64), (1, 300, 128), (37, 1000, 128), (200, 777, 64), (256, 384, 256), (65, 64 + 65, 128),
+                                    (300, 130, 128)])
+def test_causal_with_separate_lengths_is_aligned_bottom_right(variant, Nq, Nk, D):
+    """A chunk of Nq new tokens against Nk cached keys: row i sees keys 0 .. i + Nk - Nq (csrc/mask.h:53,172 of the
+    reference's CUDA tree); with fewer keys than queries the first Nq - Nk rows see nothing and come out as zeros."""
+    B, H = 2, 2
+    g = torch.Generator().manual_seed(45)
+    q = torch.randn((B, H, Nq, D), generator=g).half()
+    k = torch.randn((B, H, Nk, D), generator=g).half()
+    v = torch.randn((B, H, Nk, D), generator=g).half()
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    sm = D ** -0.5
+    if variant == "full":
+        bn = M.block_n("full", D)
+        o, lse = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), True, sm, return_lse=True)
+        ref, lse_ref = O.attention_full_int8(q8, k8, v8, qs, ks, vs, True, sm, block_n=bn, p_requant=O.p_requant_rne, return_lse=True)
+        torch.cuda.synchronize()
+        if Nk >= Nq:
+            assert_same_rounding(o, ref)
+        else:
+            assert max_abs(o, ref) <= MAX_ABS and mean_rel(o, ref) <= 2e-3
+    elif variant == "half":
+        o, lse = M.attention_int8(*gpu(q8, k8, v, qs, ks), True, sm, return_lse=True)
+        ref, lse_ref = O.attention_int8(q8, k8, v, qs, ks, True, sm, block_n=64, return_lse=True)
+        assert max_abs(o, ref) <= 4e-3 and mean_rel(o, ref) <= 5e-4
+    else:
+        o, lse = M.attention(*gpu(q, k, v), True, sm, return_lse=True)
+        ref, lse_ref = O.attention_fp(q, k, v, True, sm, block_n=64, return_lse=True)
+        assert max_abs(o, ref) <= 4e-3 and mean_rel(o, ref) <= 5e-4
+    assert torch.isfinite(o).all()
+    empty = max(Nq - Nk, 0)
+    if empty:
+        assert o[:, :, :empty].abs().max().item() == 0 and torch.isinf(lse[:, :, :empty]).all()
+    assert (lse.cpu()[:, :, empty:] - lse_ref[:, :, empty:]).abs().max().item() < 2e-3
+
+
+@pytest.mark.parametrize("variant", ["full", "fp"])
+def test_causal_separate_lengths_with_split_kv_and_per_batch_lengths(variant):
+    B, H, Nq, Nk, D = 3, 2, 150, 900, 128
+    lens = [900, 400, 150]
+    g = torch.Generator().manual_seed(46)
+    q = torch.randn((B, H, Nq, D), generator=g).half()
+    k = torch.randn((B, H, Nk, D), generator=g).half()
+    v = torch.randn((B, H, Nk, D), generator=g).half()
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    sm = D ** -0.5
+    sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    if variant == "full":
+        call = lambda **kw: M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), True, sm, seqlens_k=sl, **kw)
+        one = lambda b, n: O.attention_full_int8(q8[b:b + 1], k8[b:b + 1, :, :n], v8[b:b + 1, :, :n], qs[b:b + 1], ks[b:b + 1, :, :n],
+                                                 vs[b:b + 1], True, sm, block_n=128, p_requant=O.p_requant_rne)
+    else:
+        call = lambda **kw: M.attention(*gpu(q, k, v), True, sm, seqlens_k=sl, **kw)
+        one = lambda b, n: O.attention_fp(q[b:b + 1], k[b:b + 1, :, :n], v[b:b + 1, :, :n], True, sm, block_n=64)
+    o = call()
+    o3 = call(num_splits=3)
+    torch.cuda.synchronize()
+    for b, n in enumerate(lens):                       # every entry's mask is aligned to its own length
+        ref = one(b, n)
+        assert max_abs(o[b:b + 1], ref) <= 4e-3, (b, n)
+        assert max_abs(o3[b:b + 1], ref) <= MAX_ABS and mean_rel(o3[b:b + 1], ref) <= 3e-2, (b, n)
 
 
 # ------------------------------------------------------------------------------------------ grouped K/V heads

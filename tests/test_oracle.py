@@ -416,5 +416,36 @@ def test_separate_query_and_key_lengths_are_row_slices_of_the_square_case():
     assert torch.equal(half, O.attention_int8(q8, k8, v, qs, ks, False, 0.2, block_m=64, block_n=64)[:, :, :3])
     two = O.attention_full_int8_splitkv(q8[:, :, 70:75], k8, v8, qs[:, :, 70:75], ks, vs, False, 0.2, 2, block_m=64, block_n=64)
     assert torch.equal(two, O.attention_full_int8_splitkv(q8, k8, v8, qs, ks, vs, False, 0.2, 2, block_m=64, block_n=64)[:, :, 70:75])
-    with pytest.raises(AssertionError):
-        O.attention_full_int8(q8[:, :, :5], k8, v8, qs[:, :, :5], ks, vs, True, 0.2, block_m=64, block_n=64)
+
+
+@pytest.mark.parametrize("variant", ["full", "half", "fp"])
+@pytest.mark.parametrize("nq", [1, 37, 64, 130])
+def test_causal_with_more_keys_than_queries_is_the_tail_of_the_square_problem(variant, nq):
+    """Bottom-right aligned mask (csrc/mask.h:53,172): the last nq query rows against all N keys must equal the last nq
+    rows of the square causal evaluation, bit for bit."""
+    N = 200
+    q, k, v, _ = O.make_inputs(1, 2, N, 32, seed=18)
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    t = slice(N - nq, N)
+    kw = dict(block_m=64, block_n=64)
+    if variant == "full":
+        sq = O.attention_full_int8(q8, k8, v8, qs, ks, vs, True, 0.2, **kw)
+        part = O.attention_full_int8(q8[:, :, t], k8, v8, qs[:, :, t], ks, vs, True, 0.2, **kw)
+    elif variant == "half":
+        sq = O.attention_int8(q8, k8, v, qs, ks, True, 0.2, **kw)
+        part = O.attention_int8(q8[:, :, t], k8, v, qs[:, :, t], ks, True, 0.2, **kw)
+    else:
+        sq = O.attention_fp(q, k, v, True, 0.2, **kw)
+        part = O.attention_fp(q[:, :, t], k, v, True, 0.2, **kw)
+    assert torch.equal(part, sq[:, :, t])
+
+
+def test_causal_with_fewer_keys_than_queries_leaves_the_first_rows_empty():
+    q, k, v, _ = O.make_inputs(1, 1, 100, 16, seed=19)
+    nk = 30                                                                      # row i sees keys 0 .. i - 70
+    o, lse = O.attention_fp(q, k[:, :, :nk], v[:, :, :nk], True, 0.3, block_m=64, block_n=64, return_lse=True)
+    assert o[:, :, :70].abs().max().item() == 0 and torch.isinf(lse[:, :, :70]).all()
+    p = (q.float() @ k[:, :, :nk].float().transpose(2, 3)) * 0.3
+    keep = (torch.arange(100)[:, None] - 70) >= torch.arange(nk)[None, :]
+    want = torch.softmax(p.masked_fill(~keep, float("-inf"))[:, :, 70:], dim=-1) @ v[:, :, :nk].float()
+    assert (o[:, :, 70:].float() - want).abs().max().item() < 2e-3
