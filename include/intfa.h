@@ -139,7 +139,7 @@ const char* intfa_error_string(int code);
 /* Key-block length of a variant at a head_dim (the reference's BLOCK_N, an autotuned value there:
  * configs.py:13-19).  The running max and, on the full-int8 path, the requantisation of P advance per key block,
  * so a bit-faithful CPU evaluation must use the same value.  It holds for every shape: the kernel that takes over
- * decode-shaped calls (at most 64 query rows, no causal mask, head_dim <= 128) walks the same blocks.
+ * decode-shaped calls (at most 64 query rows, head_dim <= 128) walks the same blocks.
  * Negative INTFA_ERR_* for unknown arguments. */
 int intfa_fwd_block_n(int variant, int head_dim);
 

@@ -119,13 +119,14 @@ int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t str
     return e == hipSuccess ? INTFA_OK : (int)e;
 }
 
-// Few query rows per head and no causal mask (decoding against a cache): the full-int8 pass runs the kernel whose waves
-// share the keys of a block instead of each taking 32 query rows.
+// Few query rows per head (decoding against a cache): the full-int8 pass runs the kernel whose waves share the keys of a
+// block instead of each taking 32 query rows.
 // (Head_dim 256 stays with the general kernel: its key block is 64 there, the decode kernel's is 128, and the block
 // length is part of the arithmetic that intfa_fwd_block_n() promises.)
 constexpr int kDecodeMaxRows = 2 * kDecodeRows;
 bool decode_shaped(int variant, int seqlen, int causal, int head_dim) {
-    return variant == INTFA_VARIANT_FULL_INT8 && !causal && seqlen <= kDecodeMaxRows && head_dim <= 128;
+    (void)causal;      // the decode kernel masks too: a few new tokens against a cache
+    return variant == INTFA_VARIANT_FULL_INT8 && seqlen <= kDecodeMaxRows && head_dim <= 128;
 }
 
 int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dump_s, hipStream_t stream) {

@@ -82,7 +82,15 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
         seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
     }
     const int nb_total = (seqlen_k + BN - 1) / BN;
+    // causal: row i sees keys 0 .. i + causal_off (mask aligned to the bottom right corner as in the general kernels: a few
+    // new tokens against a cache); blocks past the last row's limit are not visited
+    const int causal_off = seqlen_k - p.seqlen;
     int nb_begin = 0, nb_end = nb_total;
+    if (p.causal) {
+        const int e = (mb * kDecodeRows + kDecodeRows + causal_off + BN - 1) / BN;
+        nb_end = e < 0 ? 0 : (e < nb_total ? e : nb_total);
+    }
+    const int causal_end = nb_end;                        // (before the split range narrows it)
     if (SPLIT) {                                           // csrc/flash_fwd_kernel.h:503-511
         nb_begin = split * p.blocks_per_split;
         const int e = nb_begin + p.blocks_per_split;
@@ -175,6 +183,10 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const uint32_t vs_rd = OFF_VS + 16 * lh;                         // + 4 * (32*dt + 8*a4) per read
     const bool own_tile0 = wave < DT;                                // head_dim 64: waves 2 and 3 own no output tile
     const int tail_keys = seqlen_k - (nb_total - 1) * BN;          // valid keys of the last block
+    // first block with a key hidden from the first row of this query block (never, without a causal mask)
+    const int diag_first = p.causal ? (mb * kDecodeRows + causal_off + 1) / BN : causal_end;
+    const int diag_begin = diag_first < 0 ? 0 : diag_first;
+    const int row_lim = p.causal ? q_row + causal_off : 0x3fffffff;   // the lane's last visible key
 
     auto step = [&](auto buf_tag, int nb) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
@@ -213,8 +225,12 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
             }
         float x[16];
         float mx = -INFINITY;
-        const bool tail = nb == nb_total - 1 && tail_keys < BN;          // wave-uniform
-        const int key_lim = tail_keys - 32 * wave - 4 * lh;              // keys of this lane with 8*a4 + b4 >= key_lim are past the end
+        // masked blocks (wave-uniform test): the ragged last block and the blocks the causal diagonal crosses
+        const bool tail = (nb == nb_total - 1 && tail_keys < BN) || nb >= diag_begin;
+        // keys of this lane with 8*a4 + b4 >= key_lim are hidden: past the end of the sequence or past the lane's row
+        const int last_key = row_lim - nb * BN < (nb == nb_total - 1 ? tail_keys : BN) - 1 ? row_lim - nb * BN
+                                                                                          : (nb == nb_total - 1 ? tail_keys : BN) - 1;
+        const int key_lim = last_key + 1 - 32 * wave - 4 * lh;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             float v = (float)sacc[r] * kk[r >> 2][r & 3];
@@ -304,7 +320,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const float l_tot = (*(const float*)(smem + xm_rd) + *(const float*)(smem + xm_rd + 128)) +
                         (*(const float*)(smem + xm_rd + 256) + *(const float*)(smem + xm_rd + 384));   // units of 1/127 when PROUND == 0
     const float vs = VBLK ? 1.f : load_scale(p.v_scale, b * p.vs_sb + hk * p.vs_sh, p.scale_dtype);
-    const bool seen = nb_begin < nb_end;         // false: an empty split range, or an empty cache entry (zeros, lse = -inf)
+    // false: an empty split range, an empty cache entry, or a causal row above the first key (zeros, lse = -inf; such a
+    // row's accumulators hold NaN from exp2(-inf - -inf), hence the selects below)
+    const bool seen = nb_begin < nb_end && m_run > -INFINITY;
     const float out_scale = !seen ? 0.f : (PROUND == 0) ? (vs / l_tot) : (vs / (127.f * l_tot));
     const float l_true = (PROUND == 0) ? l_tot * (1.f / 127.f) : l_tot;
     const float lse = seen ? m_run + __builtin_log2f(l_true) : -INFINITY;
@@ -338,12 +356,12 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
             if (OUT_DT == 0) {
                 v4h o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(o_acc[j][4 * a4 + b4] * out_scale);
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(seen ? o_acc[j][4 * a4 + b4] * out_scale : 0.f);
                 *(v4h*)(orow + d0 * 2) = o;
             } else {
                 v4s o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(o_acc[j][4 * a4 + b4] * out_scale);
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(seen ? o_acc[j][4 * a4 + b4] * out_scale : 0.f);
                 *(v4s*)(orow + d0 * 2) = o;
             }
         }

@@ -178,3 +178,52 @@ def test_per_batch_key_lengths_with_split_kv_and_argument_checks():
         M.attention_full_int8(*args, False, sm, seqlens_k=sl.long())
     with pytest.raises(ValueError):
         M.attention_full_int8(*args, False, sm, seqlens_k=sl[:2])
+
+
+# ------------------------------------------------------------------------------------------ causal decode shapes
+@pytest.mark.parametrize("B,H,H_kv,Nq,Nk,D", [
+    (2, 4, 4, 4, 1000, 128),        # four new tokens against a cache (speculative decoding)
+    (1, 2, 2, 33, 513, 128),        # two 32-row workgroups, the diagonal crosses a block boundary
+    (2, 2, 1, 64, 640, 64),
+    (1, 2, 2, 64, 64, 128),         # square: the reference's own mask
+    (1, 2, 2, 40, 25, 128),         # fewer keys than queries: the first 15 rows see nothing
+    (1, 2, 2, 1, 300, 64),          # one query: causal changes nothing
+])
+@pytest.mark.parametrize("p_round", ["rne", "reference"])
+def test_causal_decode_matches_oracle(B, H, H_kv, Nq, Nk, D, p_round):
+    x = decode_inputs(B, H, H_kv, Nq, Nk, D, seed=98)
+    sm = D ** -0.5
+    o, lse = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), True, sm, p_round=p_round,
+                                   return_lse=True)
+    torch.cuda.synchronize()
+    rep = lambda t: t.repeat_interleave(x["g"], dim=1)
+    rq = O.p_requant_rne if p_round == "rne" else O.p_requant_reference
+    ref, lse_ref = O.attention_full_int8(x["q8"], rep(x["k8"]), rep(x["v8"]), x["qs"], rep(x["ks"]), rep(x["vs"]), True, sm,
+                                         block_n=128, p_requant=rq, return_lse=True)
+    assert torch.isfinite(o).all()
+    empty = max(Nq - Nk, 0)
+    if empty:
+        assert o[:, :, :empty].abs().max().item() == 0 and torch.isinf(lse[:, :, :empty]).all()
+    assert max_abs(o, ref) <= MAX_ABS and mean_rel(o, ref) <= 2e-3
+    assert (lse.cpu()[:, :, empty:] - lse_ref[:, :, empty:]).abs().max().item() < 1e-3
+    if Nq == 1:
+        plain = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, sm, p_round=p_round)
+        assert torch.equal(o, plain)
+
+
+def test_causal_decode_with_split_kv_and_per_batch_lengths():
+    B, H, Nq, Nk, D = 3, 4, 8, 2000, 128
+    lens = [2000, 700, 8]
+    x = decode_inputs(B, H, H, Nq, Nk, D, seed=99)
+    sm = D ** -0.5
+    sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    args = gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"])
+    one = M.attention_full_int8(*args, True, sm, seqlens_k=sl)
+    split = M.attention_full_int8(*args, True, sm, seqlens_k=sl, num_splits=4)
+    torch.cuda.synchronize()
+    for b, n in enumerate(lens):
+        c = lambda t: t[b:b + 1]
+        ref = O.attention_full_int8(c(x["q8"]), c(x["k8"])[:, :, :n], c(x["v8"])[:, :, :n], c(x["qs"]), c(x["ks"])[:, :, :n],
+                                    c(x["vs"]), True, sm, block_n=128, p_requant=O.p_requant_rne)
+        assert max_abs(one[b:b + 1], ref) <= 4e-3, (b, n)
+        assert max_abs(split[b:b + 1], ref) <= MAX_ABS and mean_rel(split[b:b + 1], ref) <= 3e-2, (b, n)
