@@ -177,4 +177,29 @@ __device__ __forceinline__ float half_pair_sum(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// The reference's requantisation of P (flash_atten_full_int8.py:49-51) for two probabilities at once, in its own fp16
+// operations: fp16(p) (round to nearest even) * 127 -> fp16, + 0.5 -> fp16, truncating conversion to an integer.  The
+// multiply and the add are the packed fp16 instructions (two values each; kept apart: a fused multiply-add would skip
+// the rounding of the product); the two conversions write their byte straight into the packed word (SDWA destination
+// select), bytes B0 and B0 + 1 of pk.  B0 = 0 starts a new word.
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+template <int B0> __device__ __forceinline__ unsigned requant_p_reference2(float p0, float p1, unsigned pk) {
+    static_assert(B0 == 0 || B0 == 2, "two byte pairs per word");
+    v2h h = {(_Float16)p0, (_Float16)p1};
+    {
+#pragma clang fp contract(off)
+        h = h * (v2h){(_Float16)127.0f, (_Float16)127.0f};
+        h = h + (v2h){(_Float16)0.5f, (_Float16)0.5f};
+    }
+    const unsigned hb = __builtin_bit_cast(unsigned, h);
+    if (B0 == 0) {
+        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:WORD_0" : "=v"(pk) : "v"(hb));
+        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1" : "+v"(pk) : "v"(hb));
+    } else {
+        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0" : "+v"(pk) : "v"(hb));
+        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1" : "+v"(pk) : "v"(hb));
+    }
+    return pk;
+}
+
 }  // namespace intfa

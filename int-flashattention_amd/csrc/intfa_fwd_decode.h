@@ -253,19 +253,16 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
 #pragma unroll
         for (int w4 = 0; w4 < 4; ++w4) {
             unsigned pk = 0;
+            float e[4];
 #pragma unroll
             for (int b4 = 0; b4 < 4; ++b4) {
-                const float e = fast_exp2(fmaf(x[4 * w4 + b4], qsc, bias));      // RNE mode: 127 * p
-                lsum += e;
-                if (PROUND == 0) {
-                    pk = __builtin_amdgcn_cvt_pk_u8_f32(e, b4, pk);
-                } else {
-                    // the reference's fp16 chain: fp16(p) * 127 -> fp16, + 0.5 -> fp16, truncate (flash_atten_full_int8.py:49-51)
-                    _Float16 hp = (_Float16)e;
-                    hp = hp * (_Float16)127.0f;
-                    hp = hp + (_Float16)0.5f;
-                    pk |= (unsigned)(int)hp << (8 * b4);
-                }
+                e[b4] = fast_exp2(fmaf(x[4 * w4 + b4], qsc, bias));              // RNE mode: 127 * p
+                lsum += e[b4];
+                if (PROUND == 0) pk = __builtin_amdgcn_cvt_pk_u8_f32(e[b4], b4, pk);
+            }
+            if (PROUND != 0) {                                                   // the reference's fp16 chain
+                pk = requant_p_reference2<0>(e[0], e[1], pk);
+                pk = requant_p_reference2<2>(e[2], e[3], pk);
             }
             p8[w4] = (int)pk;
         }

@@ -373,16 +373,14 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                     }
                 } else {
                     // the reference's fp16 chain: fp16(p) * 127 -> fp16, + 0.5 -> fp16, truncate
+                    float e[4];
 #pragma unroll
                     for (int b4 = 0; b4 < 4; ++b4) {
-                        const float e = fast_exp2(fmaf(t[st][4 * w4 + b4], qsc, bias));   // p
-                        lsum += e;
-                        _Float16 hp = (_Float16)e;
-                        hp = hp * (_Float16)127.0f;
-                        hp = hp + (_Float16)0.5f;
-                        const unsigned q8 = (unsigned)(int)hp;          // truncating convert, 0..127
-                        pk |= q8 << (8 * b4);
+                        e[b4] = fast_exp2(fmaf(t[st][4 * w4 + b4], qsc, bias));          // p
+                        lsum += e[b4];
                     }
+                    pk = requant_p_reference2<0>(e[0], e[1], pk);
+                    pk = requant_p_reference2<2>(e[2], e[3], pk);
                 }
                 p8[st][w4] = (int)pk;
             }
