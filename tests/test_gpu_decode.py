@@ -227,3 +227,32 @@ def test_causal_decode_with_split_kv_and_per_batch_lengths():
                                     c(x["vs"]), True, sm, block_n=128, p_requant=O.p_requant_rne)
         assert max_abs(one[b:b + 1], ref) <= 4e-3, (b, n)
         assert max_abs(split[b:b + 1], ref) <= MAX_ABS and mean_rel(split[b:b + 1], ref) <= 3e-2, (b, n)
+
+
+@pytest.mark.parametrize("p_round,rq", [("reference", O.p_requant_reference), ("rne", O.p_requant_rne)])
+def test_causal_decode_split_matches_oracle_with_the_same_partition(p_round, rq):
+    """The decode kernel deals ceil(blocks / splits) key blocks to every split (csrc/flash_fwd_kernel.h:503) and applies
+    the causal mask inside them; the oracle evaluated over the same key ranges and merged by splitkv_combine must agree
+    to the rounding of the output (here also with blocked V scales and grouped heads)."""
+    B, H, H_kv, Nq, Nk, D, splits = 1, 8, 1, 64, 499, 128, 4
+    x = decode_inputs(B, H, H_kv, Nq, Nk, D, seed=100, v_block=256)
+    sm = D ** -0.5
+    o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), True, sm, num_splits=splits,
+                              p_round=p_round, v_scale_block=256)
+    torch.cuda.synchronize()
+    rep = lambda t: t.repeat_interleave(H // H_kv, dim=1)
+    nblk = (Nk + 127) // 128
+    per = (nblk + splits - 1) // splits
+    o_parts = torch.zeros((splits, B, H, Nq, D))
+    lse_parts = torch.full((splits, B, H, Nq), float("-inf"))
+    for s in range(splits):
+        b0, b1 = s * per, min((s + 1) * per, nblk)
+        if b0 >= b1:
+            continue
+        acc, l, m = O._blocked_forward("full", x["q8"], rep(x["k8"]), rep(x["v8"]), x["qs"], rep(x["ks"]), rep(x["vs"]), True, sm,
+                                       128, 128, key_lo=b0 * 128, key_hi=min(b1 * 128, Nk), p_requant=rq, v_scale_block=256)
+        seen = ~torch.isinf(m)
+        o_parts[s] = torch.where(seen[..., None], acc / l[..., None], torch.zeros_like(acc))
+        lse_parts[s] = torch.where(seen, m + torch.log2(l), torch.full_like(m, float("-inf")))
+    ref, _ = O.splitkv_combine(o_parts, lse_parts)
+    assert max_abs(o, ref.half()) <= 1e-3 and mean_rel(o, ref.half()) <= 1e-5
