@@ -4,8 +4,8 @@
 Prints ONE JSON line.  `value` is whole-job throughput in TOPS with the work model of the reference's harness,
 ops = 4*B*H*N^2*d (x0.5 causal; benchmark.py:90-93), inputs resident in HBM before the timed region.
 `roofline` prices the forward kernel against the dense int8 MFMA peak from per-launch HIP-event times;
-`cpu_baseline` times the CPU oracle (a port of the reference's quantised arithmetic) on the benchmark's
-CPU-runnable configuration on this box's host cores.
+`cpu_baseline` times the CPU oracle (a port of the reference's quantised arithmetic) on a bounded sample of the
+same workload - one (batch, head) slice - on this box's host cores.
 """
 import argparse
 import json
@@ -60,27 +60,45 @@ def ops_of(B, H, N, D, causal):
     return 4.0 * B * H * N * N * D * (0.5 if causal else 1.0)
 
 
-def cpu_baseline(budget_s: float):
-    """The CPU oracle on B=1, H=4, N=256, d=64, non-causal, for about `budget_s` seconds of CPU work."""
+def cpu_baseline(budget_s: float, w: dict):
+    """The CPU oracle on a bounded sample of the timed workload: one (batch, head) slice of the same shape (same N, Nk, d,
+    causal flag, variant and key-block length), for about `budget_s` seconds of CPU work.  The oracle is batched over
+    (batch, head), so the rate of one slice is the rate of the whole workload on the same cores."""
     import torch
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import intfa_oracle as O
     cores = os.cpu_count() or 1
     cores = min(cores, 16) if os.environ.get("OMP_NUM_THREADS") is None else int(os.environ["OMP_NUM_THREADS"])
     torch.set_num_threads(cores)
-    B, H, N, D = 1, 4, 256, 64
-    q, k, v, _ = O.make_inputs(B, H, N, D, seed=20)
-    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
-    fn = lambda: O.attention_full_int8(q8, k8, v8, qs, ks, vs, False, D ** -0.5, block_n=128)
-    for _ in range(3):
-        fn()
+    variant, N, D, causal = w["variant"], w["N"], w["D"], w["causal"]
+    Nk = w.get("Nk", N)
+    dt = getattr(torch, w.get("dtype", "float16"))
+    g = torch.Generator().manual_seed(20)
+    q = (torch.randn((1, 1, N, D), generator=g) * w.get("std", 1.0)).to(dt)
+    k = (torch.randn((1, 1, Nk, D), generator=g) * w.get("std", 1.0)).to(dt)
+    v = (torch.randn((1, 1, Nk, D), generator=g) * w.get("std", 1.0)).to(dt)
+    sm = D ** -0.5
+    if variant == "fp":
+        fn = lambda: O.attention_fp(q, k, v, causal, sm, block_n=64)
+    else:
+        q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k)
+        if variant == "full":
+            bn = 128 if D <= 128 else 64
+            v_block = w.get("v_block")
+            v8, vs = O.quant_perblock_channel(v, v_block) if v_block else O.quant_pertensor(v)
+            kw = dict(v_scale_block=v_block) if v_block else {}
+            fn = lambda: O.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, block_n=bn, out_dtype=dt, **kw)
+        else:
+            fn = lambda: O.attention_int8(q8, k8, v, qs, ks, causal, sm, block_n=64, out_dtype=dt)
+    fn()
     times, t_end = [], time.perf_counter() + budget_s
-    while len(times) < 10 or time.perf_counter() < t_end:
+    while len(times) < 3 or time.perf_counter() < t_end:
         t0 = time.perf_counter(); fn(); times.append(time.perf_counter() - t0)
     med = statistics.median(times)
-    return {"value": ops_of(B, H, N, D, False) / med / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(),
-            "kind": "port", "ms": med * 1e3,
-            "sample": f"{len(times)} runs of the PyTorch CPU oracle, full-int8 B{B} H{H} N{N} d{D} non-causal, median"}
+    ops = ops_of(1, 1, N, D, causal) * (Nk / N)
+    return {"value": ops / med / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port", "ms": med * 1e3,
+            "sample": f"1 of {w['B'] * w['H']} (batch, head) slices of the workload (N {N}, keys {Nk}, d {D}, "
+                      f"{'causal' if causal else 'non-causal'}, {variant}), {len(times)} runs of the PyTorch CPU oracle, median"}
 
 
 def bench_quant(args, variant, x, B, H, N, D, dt):
@@ -274,7 +292,7 @@ def main():
     if parity is not None:
         out["parity"] = parity
     if args.cpu_seconds > 0:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
+        out["cpu_baseline"] = cpu_baseline(args.cpu_seconds, w)
     print(json.dumps(out))
 
 
