@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define INTFA_VERSION 4
+#define INTFA_VERSION 5
 
 /* forward variants (one entry point each, below) */
 enum { INTFA_VARIANT_FULL_INT8 = 0, INTFA_VARIANT_HALF_INT8 = 1, INTFA_VARIANT_FP16 = 2 };
@@ -49,7 +49,7 @@ enum {
     INTFA_OK = 0,
     INTFA_ERR_NULL = -1,          /* a required pointer is NULL */
     INTFA_ERR_HEAD_DIM = -2,      /* head_dim not supported by the kernels */
-    INTFA_ERR_SEQLEN = -3,        /* seqlen not positive or seqlen_k negative */
+    INTFA_ERR_SEQLEN = -3,        /* seqlen not positive, seqlen_k negative, or causal_rows on a call it does not apply to */
     INTFA_ERR_ALIGN = -4,         /* pointer or row stride not 16-byte aligned */
     INTFA_ERR_DTYPE = -5,         /* unknown dtype enum */
     INTFA_ERR_WORKSPACE = -6,     /* workspace missing or too small for the requested split count */
@@ -128,6 +128,12 @@ typedef struct intfa_fwd_params {
                                  batch entry's length are not read.  An entry with no key gives zeros (lse = -inf).
                                  NULL = every entry has seqlen_k keys.  With causal the mask of an entry is aligned to
                                  its own length. */
+    int32_t causal_rows;      /* 0, or the number of query positions when the row axis holds several query heads of one
+                                 K/V group one after the other (decoding with grouped heads described as heads = heads_kv,
+                                 seqlen = group * positions, see heads_kv): row r is position r % causal_rows for the causal
+                                 mask.  Only with causal, full-int8, seqlen <= 64 and head_dim <= 128 (the shapes of the
+                                 decode kernel); seqlen must be a multiple of it. */
+    int32_t reserved1;        /* set to 0 */
 } intfa_fwd_params;
 
 /* Library/ABI version (INTFA_VERSION of the build). */

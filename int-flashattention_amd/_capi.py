@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libintfa.so")
 
-ABI_VERSION = 4          # INTFA_VERSION of include/intfa.h this mirror was written against
+ABI_VERSION = 5          # INTFA_VERSION of include/intfa.h this mirror was written against
 INTFA_F16, INTFA_BF16, INTFA_F32 = 0, 1, 2
 PROUND_RNE, PROUND_REFERENCE = 0, 1
 
@@ -33,7 +33,7 @@ class FwdParams(ctypes.Structure):
            ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
            ("heads_kv", ctypes.c_int32), ("seqlen_k", ctypes.c_int32),
            ("v_scale_block", ctypes.c_int32), ("reserved0", ctypes.c_int32), ("vs_stride_blk", ctypes.c_int64),
-           ("seqlens_k", ctypes.c_void_p)]
+           ("seqlens_k", ctypes.c_void_p), ("causal_rows", ctypes.c_int32), ("reserved1", ctypes.c_int32)]
     )
 
 

@@ -123,7 +123,11 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
     # Few queries per head with grouped K/V heads (decoding): the g query heads of a group become g*N rows of ONE head,
     # so that a group streams its K/V once instead of g times.  Pure re-striding: same memory, same results per row.
     g = H // H_kv
-    if g > 1 and not causal and g * N <= 2 * BLOCK and _can_fold(q_, N) and (variant == "fp" or _can_fold(q_scale, N)):
+    # (with the causal mask only where the kernel can be told the position of a row: the decode-shaped full-int8 calls)
+    fold_rows = 2 * BLOCK if not causal else (64 if variant == "full" and dk <= 128 else 0)
+    if g > 1 and g * N <= fold_rows and _can_fold(q_, N) and (variant == "fp" or _can_fold(q_scale, N)):
+        if causal:
+            p.causal_rows = N
         p.heads, p.heads_kv, p.seqlen = H_kv, H_kv, g * N
         p.q_stride_h, p.q_stride_n = g * q_.stride(1), (q_.stride(2) if N > 1 else q_.stride(1))
         p.o_stride_h = g * out.stride(1)

@@ -166,6 +166,11 @@ int run_forward(int variant, const intfa_fwd_params* p, int qk_bytes, int v_byte
     int rc = make_kparams(p, qk_bytes, v_bytes, scales, vscale, &kp);
     if (rc != INTFA_OK) return rc;
     if (variant == INTFA_VARIANT_FULL_INT8 && p->p_round != INTFA_PROUND_RNE && p->p_round != INTFA_PROUND_REFERENCE) return INTFA_ERR_DTYPE;
+    if (p->causal_rows != 0) {
+        if (p->causal_rows < 0 || !p->causal || !decode_shaped(variant, kp.seqlen, kp.causal, kp.head_dim) ||
+            kp.seqlen % p->causal_rows != 0) return INTFA_ERR_SEQLEN;
+        kp.causal_rows = p->causal_rows;
+    }
     rc = setup_split(p, block_n_for(variant, kp.head_dim), &kp);
     if (rc != INTFA_OK) return rc;
     kp.pair_mblocks = (kp.causal && kp.num_splits <= 1 && ((kp.seqlen + kBlockM - 1) / kBlockM) % 2 == 0) ? 1 : 0;
@@ -191,7 +196,7 @@ const char* intfa_error_string(int code) {
         case INTFA_OK: return "ok";
         case INTFA_ERR_NULL: return "a required pointer is NULL";
         case INTFA_ERR_HEAD_DIM: return "head_dim must be 64, 128 or 256";
-        case INTFA_ERR_SEQLEN: return "seqlen must be positive and seqlen_k not negative";
+        case INTFA_ERR_SEQLEN: return "seqlen must be positive, seqlen_k not negative, causal_rows only on causal decode-shaped full-int8 calls";
         case INTFA_ERR_ALIGN: return "pointers and row/head/batch strides must be 16-byte aligned";
         case INTFA_ERR_DTYPE: return "unknown dtype enum";
         case INTFA_ERR_WORKSPACE: return "workspace missing, misaligned or too small for num_splits";

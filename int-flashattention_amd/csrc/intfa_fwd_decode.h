@@ -84,10 +84,14 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const int nb_total = (seqlen_k + BN - 1) / BN;
     // causal: row i sees keys 0 .. i + causal_off (mask aligned to the bottom right corner as in the general kernels: a few
     // new tokens against a cache); blocks past the last row's limit are not visited
-    const int causal_off = seqlen_k - p.seqlen;
+    // (causal_rows: the rows hold several query heads of one K/V group, causal_rows positions each; a row's position is
+    // then row % causal_rows and a 32-row block can hold every position)
+    const int fold = p.causal_rows;
+    const int causal_off = seqlen_k - (fold ? fold : p.seqlen);
     int nb_begin = 0, nb_end = nb_total;
     if (p.causal) {
-        const int e = (mb * kDecodeRows + kDecodeRows + causal_off + BN - 1) / BN;
+        const int last_pos = fold ? fold : mb * kDecodeRows + kDecodeRows;       // one past the largest position in this block
+        const int e = (last_pos + causal_off + BN - 1) / BN;
         nb_end = e < 0 ? 0 : (e < nb_total ? e : nb_total);
     }
     const int causal_end = nb_end;                        // (before the split range narrows it)
@@ -184,9 +188,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const bool own_tile0 = wave < DT;                                // head_dim 64: waves 2 and 3 own no output tile
     const int tail_keys = seqlen_k - (nb_total - 1) * BN;          // valid keys of the last block
     // first block with a key hidden from the first row of this query block (never, without a causal mask)
-    const int diag_first = p.causal ? (mb * kDecodeRows + causal_off + 1) / BN : causal_end;
+    const int diag_first = p.causal ? ((fold ? 0 : mb * kDecodeRows) + causal_off + 1) / BN : causal_end;
     const int diag_begin = diag_first < 0 ? 0 : diag_first;
-    const int row_lim = p.causal ? q_row + causal_off : 0x3fffffff;   // the lane's last visible key
+    const int row_lim = p.causal ? (fold ? q_row % fold : q_row) + causal_off : 0x3fffffff;   // the lane's last visible key
 
     auto step = [&](auto buf_tag, int nb) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;

@@ -83,6 +83,9 @@ def _valid_block():
     (lambda p: (setattr(p, "v_scale_block", 128), setattr(p, "vs_stride_blk", 64)), -9),    # scale rows overlap
     (lambda p: setattr(p, "v_scale_block", -1), -9),
     (lambda p: setattr(p, "seqlen_k", -5), -3),
+    (lambda p: setattr(p, "causal_rows", 4), -3),                                            # only with causal
+    (lambda p: (setattr(p, "causal", 1), setattr(p, "causal_rows", 4)), -3),                # 256 rows: not a decode shape
+    (lambda p: (setattr(p, "causal", 1), setattr(p, "seqlen", 48), setattr(p, "causal_rows", 5)), -3),   # 48 % 5 != 0
     (lambda p: setattr(p, "seqlens_k", 0x10002), -4),
     (lambda p: (setattr(p, "v_scale_block", 128), setattr(p, "vs_stride_blk", 128), setattr(p, "v_scale", 0x10002)), -4),
 ])

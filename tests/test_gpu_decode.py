@@ -183,6 +183,9 @@ def test_per_batch_key_lengths_with_split_kv_and_argument_checks():
 # ------------------------------------------------------------------------------------------ causal decode shapes
 @pytest.mark.parametrize("B,H,H_kv,Nq,Nk,D", [
     (2, 4, 4, 4, 1000, 128),        # four new tokens against a cache (speculative decoding)
+    (2, 8, 2, 4, 1000, 128),        # grouped heads: the wrapper folds 4 heads x 4 positions into 16 rows of one K/V head
+    (1, 16, 2, 8, 700, 64),         # 8 heads x 8 positions: a 32-row block holds every position several times
+    (1, 6, 2, 5, 130, 128),         # 3 heads x 5 positions, ragged cache
     (1, 2, 2, 33, 513, 128),        # two 32-row workgroups, the diagonal crosses a block boundary
     (2, 2, 1, 64, 640, 64),
     (1, 2, 2, 64, 64, 128),         # square: the reference's own mask
