@@ -16,15 +16,12 @@
 
 namespace intfa {
 
-// Key block length of the full-int8 kernel: 128 keys, or 64 at head_dim 256 (registers and LDS).
+// Key block length of the full-int8 kernels: 128 keys, or 64 at head_dim 256 (registers and LDS).  At head_dim 256 this
+// kernel only serves the int32 S export; the forward itself is fwd_full_int8_pair_kernel (intfa_fwd_int8_pair.h), which
+// spreads the 256 output columns of a query row over two waves.
 template <int D> struct FullInt8Geom {
     static constexpr int NST = D <= 128 ? 4 : 2;
     static constexpr int BN = 32 * NST;
-    // Output columns one workgroup produces.  At head_dim 256 the 128 fp32 output registers per lane of a full-width
-    // workgroup would leave room for one wave per SIMD only, so the columns are split over two workgroups that each
-    // redo Q K^T and the softmax and multiply P with their half of V: two waves per SIMD fit again.
-    static constexpr int DV = D <= 128 ? D : 128;
-    static constexpr int NHALF = D / DV;
 };
 
 // VBLK: V carries one scale per key block and channel (layout of the reference's CUDA kernel,
@@ -34,8 +31,8 @@ template <int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUM
 __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T (32 bytes of head_dim each)
-    constexpr int DV = DUMP_S ? D : FullInt8Geom<D>::DV;       // output columns of this workgroup
-    constexpr int NHALF = D / DV;                // workgroups that share one query block (column halves)
+    static_assert(D <= 128 || DUMP_S, "head_dim 256 runs fwd_full_int8_pair_kernel");
+    constexpr int DV = D;                        // output columns
     constexpr int DT = DV / 32;                  // 32-wide output tiles along head_dim
     constexpr int NST = FullInt8Geom<D>::NST;    // 32-key sub-tiles per key block
     constexpr int BN = FullInt8Geom<D>::BN;      // keys per block
@@ -63,7 +60,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     // Causal single-pass launches pair query block i with query block n-1-i in one workgroup (heavy one first): every
     // workgroup then walks the same number of key blocks and the launch has no tail of light workgroups.
     const bool pair = CAUSAL && !SPLIT && p.pair_mblocks != 0;
-    const int per_head = (pair ? n_mblk / 2 : n_mblk * n_split) * NHALF;
+    const int per_head = pair ? n_mblk / 2 : n_mblk * n_split;
     const int n_heads = p.batch * p.heads;
     const int bid = blockIdx.x;
     // With grouped K/V heads (kv_group query heads share one K/V head) the unit dealt to an XCD is the K/V head: all
@@ -87,9 +84,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         head = bb * p.heads + hk * kv_group + r / per_head;
         rem = r % per_head;
     }
-    const int half = rem % NHALF;                // column half of this workgroup (0 when the columns are not split)
-    const int mb_idx = (rem / NHALF) / n_split;
-    const int split = (rem / NHALF) % n_split;
+    const int mb_idx = rem / n_split;
+    const int split = rem % n_split;
     const int njobs = pair ? 2 : 1;
 #pragma clang loop unroll(disable)
     for (int job = 0; job < njobs; ++job) {
@@ -149,7 +145,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
 
     // ---- global -> LDS copies (asynchronous, straight into LDS)
     const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
-    const char* Vg = DUMP_S ? Kg : p.v + b * p.v_sb + hk * p.v_sh + half * DV;
+    const char* Vg = DUMP_S ? Kg : p.v + b * p.v_sb + hk * p.v_sh;
     const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((seqlen_k - 1) * p.k_sn + D));
     const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((seqlen_k - 1) * p.v_sn + DV));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
@@ -201,7 +197,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     const int vs_c = tid - 128;
     const bool vs_thread = VBLK && vs_c >= 0 && vs_c < DV;
     // (these scales are fp32 whatever the type of the per-token scales, as in the reference's kernel)
-    const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + half * DV + (vs_thread ? vs_c : 0));
+    const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + (vs_thread ? vs_c : 0));
     auto load_vs = [&](int nb) __attribute__((always_inline)) -> float {
         if (!VBLK) return 0.f;
         const int row = p.vs_g == 1 ? nb : nb / p.vs_g;
@@ -347,7 +343,10 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         if (1 < DT) load_vfrags(vf[1], 1);
         mx = half_pair_max(mx);
         const float m_new = fmaxf(m_run, mx * qsc);
-        const float alpha = fast_exp2(m_run - m_new);
+        float alpha = fast_exp2(m_run - m_new);
+        // materialised here, well ahead of the hand-written v_fma_f32 that consumes it: the result of a transcendental
+        // needs a wait state before its first use, which the compiler inserts for its own instructions only
+        asm volatile("" : "+v"(alpha));
         m_run = m_new;
         // -------- pass 2: P = exp2(x*qsc - m), row sum, requantise
         float lsum = 0.f;
@@ -430,14 +429,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                     // o = o * alpha + pv, written as the three-operand instruction in place: left to the compiler the
                     // update is either sunk below the loop (no vector work beside the MFMAs of this stage) or, pinned
                     // here by an empty asm, emitted as v_fmac into the temporary plus a copy back (one instruction more
-                    // per output element and block).  At head_dim 256 the register allocation is tighter and the
-                    // pinned form, which leaves the choice of registers to the compiler, does not spill.
-                    if (D <= 128) {
-                        asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(o_acc[dt][r]) : "v"(alpha), "v"(pv));
-                    } else {
-                        o_acc[dt][r] = fmaf(o_acc[dt][r], alpha, pv);
-                        asm volatile("" : "+v"(o_acc[dt][r]));
-                    }
+                    // per output element and block).
+                    asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(o_acc[dt][r]) : "v"(alpha), "v"(pv));
                 }
             }
         }
@@ -519,7 +512,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     const float lse = any_key ? m_run + __builtin_log2f(l_true) : -INFINITY;
     if (SPLIT) {
         const int64_t row = ((int64_t)(split * pe->batch + eb) * e_heads + eh) * e_seqlen + q_row;
-        float* op = pe->o_part + row * D + half * DV;
+        float* op = pe->o_part + row * D;
         // a row contributes nothing to this split when the split's range is empty for its workgroup, or when every
         // block of the range lies above the row's diagonal (its wave skipped them: the running max is still -inf)
         const bool seen = nb_begin < nb_end && m_run > -INFINITY;
@@ -533,11 +526,11 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                     for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[dt][4 * a4 + b4] * out_scale : 0.f;
                     *(v4f*)(op + 32 * dt + 8 * a4 + 4 * lh) = o;
                 }
-            if (lh == 0 && half == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
+            if (lh == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
         }
         return;
     }
-    char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn + half * DV * 2;
+    char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn;
     if (q_valid) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -556,7 +549,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                 *(v4s*)(orow + d0 * 2) = o;
             }
         }
-    if (pe->lse != nullptr && lh == 0 && half == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
+    if (pe->lse != nullptr && lh == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
     }   // q_valid
     }   // job
 #endif  // __HIP_DEVICE_COMPILE__
