@@ -36,6 +36,8 @@ WORKLOADS = {
                                              dtype="bfloat16", std=0.5),
     "full_int8_B16_H16_N1024_d256_bf16": dict(variant="full", B=16, H=16, N=1024, D=256, causal=False, splits=1,
                                               dtype="bfloat16", std=0.5),
+    # head_dim 256 at the headline's batch, heads and length (the eight-wave kernel of that head_dim)
+    "full_int8_B4_H32_N4096_d256": dict(variant="full", B=4, H=32, N=4096, D=256, causal=False, splits=1),
     # the headline shape with V quantised per block of 128 keys and channel (the V scales of the reference's CUDA kernel)
     "full_int8_B4_H32_N4096_d128_vblock": dict(variant="full", B=4, H=32, N=4096, D=128, causal=False, splits=1, v_block=128),
     # decoding against a cache: one query per head, 16384 cached keys (HBM-bound: K and V are streamed once)

@@ -85,6 +85,9 @@ template <int ROW_BYTES> __device__ __forceinline__ int swz_k(int row) {
 }
 // int8 V rows read by ds_read_b64_tr_b8: a 16-lane group touches rows {0,1,2,3,8,9,10,11} + 4h of a sub-tile.
 template <int ROW_BYTES> __device__ __forceinline__ int swz_v8(int row) {
+    // 256-byte rows all start at bank 0, and the two 16-lane groups served together read neighbouring chunks (2 dt and
+    // 2 dt + 1) of eight rows each: even flips keep the groups in the even and the odd chunks respectively
+    if (ROW_BYTES >= 256) return 2 * ((row & 3) | ((row >> 1) & 4));
     if (ROW_BYTES >= 128) return (row & 3) | ((row >> 1) & 4);
     return ((row >> 1) & 1) | ((row >> 2) & 2);
 }

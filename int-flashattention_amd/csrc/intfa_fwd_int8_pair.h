@@ -176,12 +176,12 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
     // V (A operand of O^T = V^T P^T) through the transposing 8-byte load; this wave's columns start at chunk 8 hf
     const int g16 = lane >> 4, i16 = lane & 15, jj = i16 >> 1;
     const int v_row0 = 8 * (jj >> 2) + 4 * lh + (jj & 3);
-    const int v_swz = swz_v8<D>(v_row0) & 7;
+    const int v_swz = swz_v8<D>(v_row0) & 15;
     uint32_t v_rd[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-        const int c = 2 * dt + (g16 & 1);
-        v_rd[dt] = OFF_V + v_row0 * D + 8 * (i16 & 1) + ((c ^ v_swz) << 4) + DVW * hf;
+        const int c = 8 * hf + 2 * dt + (g16 & 1);
+        v_rd[dt] = OFF_V + v_row0 * D + 8 * (i16 & 1) + ((c ^ v_swz) << 4);
     }
     const uint32_t v_own = 32 * hf * D, v_oth = 32 * (hf ^ 1) * D;      // sub-tile of this wave's P, of the partner's
     const uint32_t ks_rd = OFF_KS + 4 * 32 * hf + 16 * lh;              // + 32 * a4 per read

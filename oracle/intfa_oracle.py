@@ -337,7 +337,7 @@ def splitkv_ranges_causal(n_keys: int, block_m: int, block_n: int, num_splits: i
 
 def attention_full_int8_splitkv(q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float, num_splits: int, *,
                                 block_m: int = 128, block_n: int = 128, out_dtype=torch.float16,
-                                v_scale_block: Optional[int] = None):
+                                v_scale_block: Optional[int] = None, p_requant=p_requant_reference):
     """Full-int8 forward evaluated as ``num_splits`` independent key ranges merged by ``splitkv_combine``: the ranges of
     ``splitkv_ranges`` for a non-causal pass, those of ``splitkv_ranges_causal`` (per row tile) for a causal one."""
     B, H, N, D = q.shape
@@ -354,7 +354,7 @@ def attention_full_int8_splitkv(q, k, v, q_scale, k_scale, v_scale, causal: bool
             continue
         acc, l, m = _blocked_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale,
                                      block_m, block_n, key_lo=b0 * block_n, key_hi=min(b1 * block_n, k.shape[2]),
-                                     row_lo=r0, row_hi=r1, v_scale_block=v_scale_block)
+                                     row_lo=r0, row_hi=r1, v_scale_block=v_scale_block, p_requant=p_requant)
         seen = ~torch.isinf(m[:, :, r0:r1])          # rows above the split's range saw no key
         a, ll, mm = acc[:, :, r0:r1], l[:, :, r0:r1], m[:, :, r0:r1]
         o_parts[s, :, :, r0:r1] = torch.where(seen[..., None], a / ll[..., None], torch.zeros_like(a))
