@@ -52,9 +52,9 @@ WORKLOADS = {
 # what the same counter reads for a plain copy of known size; None where not measured.
 MEASURED_TRAFFIC_BYTES = {
     # FETCH_SIZE x 1.9997 + WRITE_SIZE x 1.0 (KiB per dispatch, factors from a 256 MiB copy): 194.2 MiB read + 128 MiB written
-    "full_int8_B4_H32_N4096_d128": 337860823,
+    "full_int8_B4_H32_N4096_d128": 337902723,
     # FETCH_SIZE 528548.6 x 1.9998 + WRITE_SIZE 256 x 1.0: 1032.2 MiB read + 0.25 MiB written (algorithmic: 1082523648)
-    "full_int8_decode_B32_H32_Nq1_Nk4096_d128": 1082610029,
+    "full_int8_decode_B32_H32_Nq1_Nk4096_d128": 1082605181,
 }
 
 
