@@ -219,7 +219,7 @@ int intfa_fwd_suggest_splits(const intfa_fwd_params* p, int variant, int num_cus
     const int64_t slots = 2ll * cus;                                           // two workgroups per compute unit
     int64_t wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kBlockM - 1) / kBlockM);
     if (decode_shaped(variant, p->seqlen, p->causal, p->head_dim)) wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kDecodeRows - 1) / kDecodeRows);
-    else if (variant == INTFA_VARIANT_FULL_INT8 && p->head_dim == 256) wgs *= 2;     // eight-wave workgroups, one per compute unit
+    else if (p->head_dim == 256) wgs *= 2;     // full-int8: eight-wave workgroups, one per compute unit; the others: column halves
     if (wgs * 5 >= slots * 4) return 1;                                        // at least 80 % of the slots are used anyway
     const int seqlen_k = p->seqlen_k > 0 ? p->seqlen_k : p->seqlen;
     const int bn = block_n_for(variant, p->head_dim);

@@ -29,14 +29,23 @@ __device__ __forceinline__ v8bf pack_p_bf16(const float* e) {
 
 // QK_INT8: int8 Q/K with scales (half-int8) or 16-bit Q/K (fp16/bf16 variant).  IO_DT: type of V, P and the output
 // (and of Q/K when !QK_INT8): 0 fp16, 1 bf16.
+// Output columns one workgroup produces.  At head_dim 256 a full-width workgroup needs 128 fp32 output registers per lane:
+// one wave per SIMD and spills.  The columns are split over two workgroups that each redo Q K^T and the softmax and
+// multiply P with their half of V.
+template <int D> struct F16PvGeom {
+    static constexpr int DV = D <= 128 ? D : 128;
+    static constexpr int NHALF = D / DV;
+};
+
 template <bool QK_INT8, int D, bool CAUSAL, int IO_DT, bool SPLIT>
-__global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel(const KParams p) {
+__global__ void __launch_bounds__(kThreads, 2) fwd_f16pv_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr int BN = kBlockN16, NST = BN / 32;
     constexpr int QB = QK_INT8 ? 1 : 2;               // bytes per Q/K element
-    constexpr int KROW = D * QB, VROW = D * 2;        // bytes per K / V row
+    constexpr int DV = F16PvGeom<D>::DV, NHALF = F16PvGeom<D>::NHALF;
+    constexpr int KROW = D * QB, VROW = DV * 2;       // bytes per K row / per V row of this workgroup's columns
     constexpr int KS = KROW / 32;                     // MFMA k-steps of S^T (32 bytes of a row each)
-    constexpr int DT = D / 32;                        // 32-wide output tiles
+    constexpr int DT = DV / 32;                       // 32-wide output tiles
     constexpr int KT = BN * KROW, VT = BN * VROW;
     constexpr int KCH = KROW / 16, VCH = VROW / 16;
     constexpr int OFF_KS = 0;
@@ -54,7 +63,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     // Causal single-pass launches pair query block i with query block n-1-i in one workgroup (heavy one first): every
     // workgroup then walks the same number of key blocks and the launch has no tail of light workgroups.
     const bool pair = CAUSAL && !SPLIT && p.pair_mblocks != 0;
-    const int per_head = pair ? n_mblk / 2 : n_mblk * n_split;
+    const int per_head = (pair ? n_mblk / 2 : n_mblk * n_split) * NHALF;
     const int n_heads = p.batch * p.heads;
     const int bid = blockIdx.x;
     // With grouped K/V heads (kv_group query heads share one K/V head) the unit dealt to an XCD is the K/V head: all
@@ -78,8 +87,9 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
         head = bb * p.heads + hk * kv_group + r / per_head;
         rem = r % per_head;
     }
-    const int mb_idx = rem / n_split;
-    const int split = rem % n_split;
+    const int half = rem % NHALF;                // column half of this workgroup (0 when the columns are not split)
+    const int mb_idx = (rem / NHALF) / n_split;
+    const int split = (rem / NHALF) % n_split;
     const int njobs = pair ? 2 : 1;
 #pragma clang loop unroll(disable)
     for (int job = 0; job < njobs; ++job) {
@@ -135,7 +145,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
 
     // ---- global -> LDS copies
     const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
-    const char* Vg = p.v + b * p.v_sb + hk * p.v_sh;
+    const char* Vg = p.v + b * p.v_sb + hk * p.v_sh + half * DV * 2;
     const v4i k_rsrc = make_rsrc(Kg, (uint32_t)((seqlen_k - 1) * p.k_sn + KROW));
     const v4i v_rsrc = make_rsrc(Vg, (uint32_t)((seqlen_k - 1) * p.v_sn + VROW));
     const uint32_t k_sn = (uint32_t)p.k_sn, v_sn = (uint32_t)p.v_sn;
@@ -370,7 +380,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
     const float lse = any_key ? m_run + __builtin_log2f(l_tot) : -INFINITY;
     if (SPLIT) {
         const int64_t row = ((int64_t)(split * pe->batch + eb) * e_heads + eh) * e_seqlen + q_row;
-        float* op = pe->o_part + row * D;
+        float* op = pe->o_part + row * D + half * DV;
         // a row contributes nothing to this split when the split's range is empty for its workgroup, or when every
         // block of the range lies above the row's diagonal (its wave skipped them: the running max is still -inf)
         const bool seen = nb_begin < nb_end && m_run > -INFINITY;
@@ -384,11 +394,11 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
                     for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[dt][4 * a4 + b4] * inv : 0.f;
                     *(v4f*)(op + 32 * dt + 8 * a4 + 4 * lh) = o;
                 }
-            if (lh == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
+            if (lh == 0 && half == 0) pe->lse_part[row] = seen ? lse : -INFINITY;
         }
         return;
     }
-    char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn;
+    char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn + half * DV * 2;
     if (q_valid) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -407,7 +417,7 @@ __global__ void __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) fwd_f16pv_kernel
                 *(v4s*)(orow + d0 * 2) = o;
             }
         }
-    if (pe->lse != nullptr && lh == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
+    if (pe->lse != nullptr && lh == 0 && half == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
     }   // q_valid
     }   // job
 #endif  // __HIP_DEVICE_COMPILE__

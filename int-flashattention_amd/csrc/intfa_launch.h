@@ -17,8 +17,10 @@ struct LaunchSel {
 };
 
 // One workgroup per (batch, head, 128-row query block, split); causal single-pass launches pair the query blocks.
-template <typename K> inline int launch_kernel(K kernel, const KParams& kp, hipStream_t stream, int threads = kThreads) {
-    const int grid = kp.batch * kp.heads * ((kp.seqlen + kBlockM - 1) / kBlockM) * kp.num_splits / (kp.pair_mblocks ? 2 : 1);
+// `column_halves`: workgroups per query block (2 where a kernel splits the output columns over two workgroups).
+template <typename K> inline int launch_kernel(K kernel, const KParams& kp, hipStream_t stream, int threads = kThreads,
+                                               int column_halves = 1) {
+    const int grid = kp.batch * kp.heads * ((kp.seqlen + kBlockM - 1) / kBlockM) * kp.num_splits / (kp.pair_mblocks ? 2 : 1) * column_halves;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), 0, stream, kp);
     return (int)hipGetLastError();
 }
