@@ -166,11 +166,17 @@ def test_split_kv_matches_oracle_split(causal, splits):
     assert abs(mean_rel(o, single) - mean_rel(ref, single)) <= 1e-3
 
 
-def test_split_kv_head_dim_256():
-    x = quantised(1, 2, 512, 256, seed=18)
+@pytest.mark.parametrize("n,causal,splits,p_round", [(512, False, 2, "reference"), (512, True, 3, "reference"),
+                                                    (512, False, 4, "rne"), (700, False, 3, "rne"), (640, True, 2, "rne")])
+def test_split_kv_head_dim_256(n, causal, splits, p_round):
+    """The head_dim 256 kernel (two waves per 32 query rows) against the oracle evaluated over the same key ranges, for
+    both roundings of P: with the partition matched, only fp32 summation order and the output rounding are left."""
+    x = quantised(1, 2, n, 256, seed=18)
     sm = 256 ** -0.5
-    o = run_full(x, False, sm, num_splits=2, p_round="reference")
-    ref = O.attention_full_int8_splitkv(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], False, sm, 2, block_n=64)
+    o = run_full(x, causal, sm, num_splits=splits, p_round=p_round)
+    rq = O.p_requant_rne if p_round == "rne" else O.p_requant_reference
+    ref = O.attention_full_int8_splitkv(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, splits, block_n=64,
+                                        p_requant=rq)
     assert max_abs(o, ref) <= 4e-3 and mean_rel(o, ref) <= 2e-4
 
 
@@ -183,6 +189,8 @@ HALF_FP_CASES = [
     (2, 3, 384, 64, True, torch.float16),
     (1, 2, 256, 256, False, torch.float16),
     (1, 2, 384, 256, True, torch.float16),
+    (2, 3, 300, 256, False, torch.bfloat16),     # ragged length, column halves
+    (1, 2, 641, 256, True, torch.float16),
     (1, 2, 512, 128, True, torch.bfloat16),
     (2, 2, 256, 64, False, torch.bfloat16),
 ]
