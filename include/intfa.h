@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define INTFA_VERSION 5
+#define INTFA_VERSION 6
 
 /* forward variants (one entry point each, below) */
 enum { INTFA_VARIANT_FULL_INT8 = 0, INTFA_VARIANT_HALF_INT8 = 1, INTFA_VARIANT_FP16 = 2 };
@@ -204,6 +204,36 @@ int intfa_quant_pertensor(const void* x, int64_t stride_b, int64_t stride_h, int
 int intfa_quant_perblock_channel(const void* x, int64_t stride_b, int64_t stride_h, int64_t stride_n, void* q8, float* scale,
                                  int32_t batch, int32_t heads, int32_t seqlen, int32_t head_dim, int32_t block,
                                  int32_t dtype, void* stream);
+
+/* Appends new keys (and values) to an int8 K/V cache: the counterpart, for the quantised cache this library reads, of
+ * the copy the reference's cache kernel makes of knew/vnew before it attends (csrc/flash_fwd_kernel.h:690-790,
+ * Append_KV; csrc/flash.h:104-112; rotary embedding and paged caches are not part of this build).  For batch entry b the
+ * rows go to positions len_b .. len_b + seqlen_new - 1 of the cache, len_b = seqlens_k[b] (device memory, clamped to
+ * [0, seqlen_cache]) or seqlen_filled when seqlens_k is NULL; rows that would land at or past seqlen_cache are dropped.
+ * The lengths themselves are the caller's to advance (a forward call with seqlens_k = len + seqlen_new then sees them).
+ *   K: quantised per token exactly as intfa_quant_pertoken does (scale = absmax / 127 in k_new's type, stored into
+ *      k_scale_cache at the row's position);
+ *   V: quantised with the cache's existing scale v_scale[b, h] (V has one scale per (batch, head), which an append
+ *      cannot change): q = round-half-even(v / scale) in v_new's type, saturated to [-127, 127].  v_new = NULL: K only.
+ * k_new, v_new: [batch, heads_kv, seqlen_new, head_dim] fp16 or bf16 (dtype), head_dim contiguous, strides in elements;
+ * k_cache, v_cache: int8 [batch, heads_kv, seqlen_cache, head_dim], head_dim contiguous, row strides multiples of 8;
+ * k_scale_cache: [batch, heads_kv, seqlen_cache] and v_scale: [batch, heads_kv], both in k_new's type. */
+typedef struct intfa_append_params {
+    const void* k_new; const void* v_new;
+    int64_t kn_stride_b, kn_stride_h, kn_stride_n;
+    int64_t vn_stride_b, vn_stride_h, vn_stride_n;
+    void* k_cache; void* v_cache;
+    int64_t kc_stride_b, kc_stride_h, kc_stride_n;
+    int64_t vc_stride_b, vc_stride_h, vc_stride_n;
+    void* k_scale_cache;
+    int64_t ksc_stride_b, ksc_stride_h, ksc_stride_n;
+    const void* v_scale;
+    int64_t vs_stride_b, vs_stride_h;
+    const int32_t* seqlens_k;
+    int32_t seqlen_filled;
+    int32_t batch, heads_kv, seqlen_new, seqlen_cache, head_dim, dtype;
+} intfa_append_params;
+int intfa_kvcache_append_int8(const intfa_append_params* p, void* stream);
 
 #ifdef __cplusplus
 }

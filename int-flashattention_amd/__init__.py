@@ -11,7 +11,7 @@ from .flash_atten_fp import attention
 from .flash_atten_int8 import attention_int8
 from .flash_atten_full_int8 import attention_full_int8
 from ._host import debug_qk_int32, block_n
-from .quant import quant_pertoken, quant_pertensor, quant_perblock_channel
+from .quant import quant_pertoken, quant_pertensor, quant_perblock_channel, kvcache_append
 
 __all__ = ["attention", "attention_int8", "attention_full_int8", "debug_qk_int32", "block_n", "quant_pertoken", "quant_pertensor",
-           "quant_perblock_channel"]
+           "quant_perblock_channel", "kvcache_append"]

@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libintfa.so")
 
-ABI_VERSION = 5          # INTFA_VERSION of include/intfa.h this mirror was written against
+ABI_VERSION = 6          # INTFA_VERSION of include/intfa.h this mirror was written against
 INTFA_F16, INTFA_BF16, INTFA_F32 = 0, 1, 2
 PROUND_RNE, PROUND_REFERENCE = 0, 1
 
@@ -37,12 +37,27 @@ class FwdParams(ctypes.Structure):
     )
 
 
+class AppendParams(ctypes.Structure):
+    """Mirror of ``intfa_append_params`` (include/intfa.h)."""
+    _fields_ = (
+        [("k_new", ctypes.c_void_p), ("v_new", ctypes.c_void_p)]
+        + [(n, ctypes.c_int64) for n in ("kn_stride_b", "kn_stride_h", "kn_stride_n", "vn_stride_b", "vn_stride_h", "vn_stride_n")]
+        + [("k_cache", ctypes.c_void_p), ("v_cache", ctypes.c_void_p)]
+        + [(n, ctypes.c_int64) for n in ("kc_stride_b", "kc_stride_h", "kc_stride_n", "vc_stride_b", "vc_stride_h", "vc_stride_n")]
+        + [("k_scale_cache", ctypes.c_void_p)]
+        + [(n, ctypes.c_int64) for n in ("ksc_stride_b", "ksc_stride_h", "ksc_stride_n")]
+        + [("v_scale", ctypes.c_void_p), ("vs_stride_b", ctypes.c_int64), ("vs_stride_h", ctypes.c_int64),
+           ("seqlens_k", ctypes.c_void_p)]
+        + [(n, ctypes.c_int32) for n in ("seqlen_filled", "batch", "heads_kv", "seqlen_new", "seqlen_cache", "head_dim", "dtype")]
+    )
+
+
 VARIANT_FULL_INT8, VARIANT_HALF_INT8, VARIANT_FP16 = 0, 1, 2
 
 EXPORTS = ("intfa_version", "intfa_error_string", "intfa_fwd_block_n", "intfa_fwd_workspace_bytes", "intfa_fwd_suggest_splits",
            "intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16", "intfa_debug_qk_int32",
            "intfa_quant_pertoken", "intfa_quant_pertensor_workspace_bytes", "intfa_quant_pertensor",
-           "intfa_quant_perblock_channel")
+           "intfa_quant_perblock_channel", "intfa_kvcache_append_int8")
 
 _lib = None
 
@@ -83,6 +98,8 @@ def load():
     lib.intfa_quant_pertensor.argtypes = [vp, i64, i64, i64, vp, vp, i32, i32, i32, i32, i32, vp, ctypes.c_size_t, vp]
     lib.intfa_quant_perblock_channel.restype = ctypes.c_int
     lib.intfa_quant_perblock_channel.argtypes = [vp, i64, i64, i64, vp, vp, i32, i32, i32, i32, i32, i32, vp]
+    lib.intfa_kvcache_append_int8.restype = ctypes.c_int
+    lib.intfa_kvcache_append_int8.argtypes = [ctypes.POINTER(AppendParams), vp]
     if lib.intfa_version() != ABI_VERSION:
         raise RuntimeError(f"{LIB_PATH} has ABI version {lib.intfa_version()}, this package expects {ABI_VERSION}: rebuild it")
     _lib = lib

@@ -292,6 +292,74 @@ int grid_for(int64_t rows, int rows_per_block) {
     return (int)(blocks < cap ? blocks : cap);
 }
 
+// ---- append to an int8 K/V cache: one row of new keys or values per LPR lanes, written at the row's position in the
+// cache.  IS_V: the scale is the cache's (given), the quotient saturates; else the row's own scale, stored beside it.
+struct AppendSide {
+    const char* x; char* cache; char* scale;      // scale: k_scale_cache (written) or v_scale (read)
+    int64_t xb, xh, xn;                           // bytes
+    int64_t cb, ch, cn;                           // bytes (int8 elements)
+    int64_t sb, sh, sn;                           // scale strides, elements (sn unused for V)
+};
+struct AppendParams {
+    AppendSide k, v;
+    const int32_t* seqlens_k;
+    int32_t seqlen_filled, heads, seqlen_new, seqlen_cache, head_dim;
+    int64_t rows;                                 // batch * heads * seqlen_new
+};
+
+template <int DT, int LPR, bool IS_V> __global__ void __launch_bounds__(256) kv_append_kernel(const AppendParams p) {
+    constexpr int RPB = 256 / LPR;
+    const AppendSide& s = IS_V ? p.v : p.k;
+    const int sub = threadIdx.x % LPR, rl = threadIdx.x / LPR;
+    const uint32_t step = gridDim.x * RPB, rows = (uint32_t)p.rows;
+    // (the trip count depends on the workgroup only through rl, and rows is a multiple of nothing: the lanes of a row
+    // share rl, so they enter and leave the loop together and the shuffles below see all of them)
+    for (uint32_t row = blockIdx.x * RPB + rl; row < rows; row += step) {
+        const uint32_t bh = row / (uint32_t)p.seqlen_new, i = row - bh * (uint32_t)p.seqlen_new;
+        const uint32_t b = bh / (uint32_t)p.heads, h = bh - b * (uint32_t)p.heads;
+        int len = p.seqlen_filled;
+        if (p.seqlens_k != nullptr) {
+            const int n = p.seqlens_k[b];
+            len = n < 0 ? 0 : (n < p.seqlen_cache ? n : p.seqlen_cache);
+        }
+        const int64_t pos = (int64_t)len + i;
+        const v4i raw = *(const v4i*)(s.x + b * s.xb + h * s.xh + i * s.xn + sub * 16);
+        uint16_t sbits;
+        if (IS_V) {
+            sbits = ((const uint16_t*)s.scale)[b * s.sb + h * s.sh];
+        } else {
+            uint32_t m = amax8(raw);
+#pragma unroll
+            for (int off = LPR / 2; off > 0; off >>= 1) {
+                const uint32_t o = (uint32_t)__shfl_xor((int)m, off, 64);
+                m = m > o ? m : o;
+            }
+            sbits = from_f32<DT>(to_f32<DT>((uint16_t)m) / 127.0f);
+        }
+        if (pos >= p.seqlen_cache) continue;                                   // no room: the row is dropped
+        char* dst = s.cache + b * s.cb + h * s.ch + pos * s.cn + sub * 8;
+        const RowDivisor d = make_divisor(to_f32<DT>(sbits));
+        if (IS_V) {
+            int out[2];
+#pragma unroll
+            for (int w = 0; w < 2; ++w) {
+                float q[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t word = (uint32_t)raw[2 * w + j / 2];
+                    const float t = quotient16<DT>((uint16_t)(j & 1 ? word >> 16 : word & 0xffffu), d);
+                    q[j] = t != t ? t : __builtin_fminf(__builtin_fmaxf(t, -127.0f), 127.0f);      // (NaN from 0 / 0 stays NaN: byte 0)
+                }
+                out[w] = (int)pack4_rne(q[0], q[1], q[2], q[3]);
+            }
+            *(v2i*)dst = (v2i){out[0], out[1]};
+        } else {
+            if (sub == 0) ((uint16_t*)s.scale)[b * s.sb + h * s.sh + pos * s.sn] = sbits;
+            quant_store8<DT>(raw, d, dst);
+        }
+    }
+}
+
 }  // namespace
 
 #define INTFA_LPR_SWITCH(d, CALL)            \
@@ -365,6 +433,52 @@ int intfa_quant_perblock_channel(const void* x, int64_t stride_b, int64_t stride
         if (dtype == INTFA_F16) hipLaunchKernelGGL((quant_blockchan_kernel<0, LPR>), dim3((int)grid), dim3(256), 0, st, qp, block, nblk, scale); \
         else hipLaunchKernelGGL((quant_blockchan_kernel<1, LPR>), dim3((int)grid), dim3(256), 0, st, qp, block, nblk, scale); } while (0)
     INTFA_LPR_SWITCH(head_dim, INTFA_CALL)
+#undef INTFA_CALL
+    return (int)hipGetLastError();
+}
+
+int intfa_kvcache_append_int8(const intfa_append_params* a, void* stream) {
+    if (a == nullptr || a->k_new == nullptr || a->k_cache == nullptr || a->k_scale_cache == nullptr) return INTFA_ERR_NULL;
+    const bool with_v = a->v_new != nullptr;
+    if (with_v && (a->v_cache == nullptr || a->v_scale == nullptr)) return INTFA_ERR_NULL;
+    if (a->batch <= 0 || a->heads_kv <= 0) return INTFA_ERR_SHAPE;
+    if (a->seqlen_new <= 0 || a->seqlen_cache <= 0 ||
+        (a->seqlens_k == nullptr && (a->seqlen_filled < 0 || a->seqlen_filled > a->seqlen_cache))) return INTFA_ERR_SEQLEN;
+    const int d = a->head_dim;
+    if (d != 16 && d != 32 && d != 64 && d != 128 && d != 256) return INTFA_ERR_HEAD_DIM;
+    if (a->dtype != INTFA_F16 && a->dtype != INTFA_BF16) return INTFA_ERR_DTYPE;
+    const int64_t rows = (int64_t)a->batch * a->heads_kv * a->seqlen_new;
+    if (rows >= (1ll << 31) - (1 << 24)) return INTFA_ERR_SHAPE;
+    // 16-byte loads of the 16-bit rows (strides in elements: multiples of 8), 8-byte stores of the int8 rows
+    auto misaligned = [](const void* ptr, int64_t s0, int64_t s1, int64_t s2, unsigned bytes) {
+        return (reinterpret_cast<uintptr_t>(ptr) & (bytes - 1u)) != 0 || s0 % 8 || s1 % 8 || s2 % 8;
+    };
+    if (misaligned(a->k_new, a->kn_stride_b, a->kn_stride_h, a->kn_stride_n, 16) ||
+        misaligned(a->k_cache, a->kc_stride_b, a->kc_stride_h, a->kc_stride_n, 8)) return INTFA_ERR_ALIGN;
+    if (with_v && (misaligned(a->v_new, a->vn_stride_b, a->vn_stride_h, a->vn_stride_n, 16) ||
+                   misaligned(a->v_cache, a->vc_stride_b, a->vc_stride_h, a->vc_stride_n, 8))) return INTFA_ERR_ALIGN;
+    if ((reinterpret_cast<uintptr_t>(a->k_scale_cache) & 1u) || (with_v && (reinterpret_cast<uintptr_t>(a->v_scale) & 1u)) ||
+        (a->seqlens_k != nullptr && (reinterpret_cast<uintptr_t>(a->seqlens_k) & 3u))) return INTFA_ERR_ALIGN;
+    if (a->kn_stride_n < d || a->kc_stride_n < d || (with_v && (a->vn_stride_n < d || a->vc_stride_n < d))) return INTFA_ERR_SHAPE;
+    AppendParams ap;
+    ap.k = {(const char*)a->k_new, (char*)a->k_cache, (char*)a->k_scale_cache, a->kn_stride_b * 2, a->kn_stride_h * 2,
+            a->kn_stride_n * 2, a->kc_stride_b, a->kc_stride_h, a->kc_stride_n, a->ksc_stride_b, a->ksc_stride_h, a->ksc_stride_n};
+    ap.v = {(const char*)a->v_new, (char*)a->v_cache, (char*)const_cast<void*>(a->v_scale), a->vn_stride_b * 2, a->vn_stride_h * 2,
+            a->vn_stride_n * 2, a->vc_stride_b, a->vc_stride_h, a->vc_stride_n, a->vs_stride_b, a->vs_stride_h, 0};
+    ap.seqlens_k = a->seqlens_k;
+    ap.seqlen_filled = a->seqlen_filled;
+    ap.heads = a->heads_kv; ap.seqlen_new = a->seqlen_new; ap.seqlen_cache = a->seqlen_cache; ap.head_dim = d;
+    ap.rows = rows;
+    hipStream_t st = (hipStream_t)stream;
+#define INTFA_CALL(LPR) do { const int g = grid_for(rows, 256 / LPR); \
+        if (a->dtype == INTFA_F16) { \
+            hipLaunchKernelGGL((kv_append_kernel<0, LPR, false>), dim3(g), dim3(256), 0, st, ap); \
+            if (with_v) hipLaunchKernelGGL((kv_append_kernel<0, LPR, true>), dim3(g), dim3(256), 0, st, ap); \
+        } else { \
+            hipLaunchKernelGGL((kv_append_kernel<1, LPR, false>), dim3(g), dim3(256), 0, st, ap); \
+            if (with_v) hipLaunchKernelGGL((kv_append_kernel<1, LPR, true>), dim3(g), dim3(256), 0, st, ap); \
+        } } while (0)
+    INTFA_LPR_SWITCH(d, INTFA_CALL)
 #undef INTFA_CALL
     return (int)hipGetLastError();
 }

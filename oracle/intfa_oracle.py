@@ -48,6 +48,9 @@ How every function is pinned (tests/test_oracle.py):
 * blocked V scales: a 4-D scale tensor filled with one value per (batch, head) reproduces the scalar form bit for
   bit; the result equals the scalar form applied to V pre-multiplied by the block/channel factors when these are
   powers of two; ``quant_perblock_channel`` against a pure-Python loop, and every (block, channel) reaches +-127.
+* ``kvcache_append``: a cache filled by two appends equals the quantisers applied to the concatenation (K: rows are
+  independent, bit for bit incl. scales; V: with the concatenation's per-tensor scale, bit for bit); values beyond the
+  cache's V scale saturate at +-127; rows outside the appended range stay untouched; rows past the end are dropped.
 
 The reference holds no golden vectors for this path (its only test asserts the fp16 forward with
 atol=1e-2, benchmark.py:242), so none are used.
@@ -80,6 +83,27 @@ def quant_pertensor(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     x_scale = x_max / 127
     ret = torch.round(x / x_scale[:, :, None, None]).to(torch.int8)
     return ret, x_scale
+
+
+def kvcache_append(k_cache, k_scale_cache, k_new, seqlens_k, v_cache=None, v_scale=None, v_new=None) -> None:
+    """Appends new keys (and values) to an int8 K/V cache in place: for batch entry b the rows go to positions
+    len_b .. len_b + N_new - 1, len_b = seqlens_k[b] clamped to the cache (the copy of knew/vnew that the reference's
+    cache kernel makes, csrc/flash_fwd_kernel.h:690-790, for a quantised cache); rows past the end of the cache are
+    dropped.  K rows are quantised per token (``quant_pertoken``: the rows are independent, so this equals quantising
+    the concatenation), their scales go to ``k_scale_cache``; V rows with the cache's existing per-(batch, head) scale,
+    q = round-half-even(v / scale) in v's dtype saturated to [-127, 127] (0 / 0 gives 0)."""
+    Z, _, n_new, _ = k_new.shape
+    n_cache = k_cache.shape[2]
+    k8, ks = quant_pertoken(k_new)
+    for b in range(Z):
+        n0 = min(max(int(seqlens_k[b]), 0), n_cache)
+        n = min(n_new, n_cache - n0)
+        k_cache[b, :, n0:n0 + n] = k8[b, :, :n]
+        k_scale_cache[b, :, n0:n0 + n] = ks[b, :, :n]
+        if v_new is not None:
+            q = torch.round(v_new[b, :, :n] / v_scale[b][:, None, None])
+            q = torch.where(torch.isnan(q), torch.zeros_like(q), q.clamp(-127, 127))
+            v_cache[b, :, n0:n0 + n] = q.to(torch.int8)
 
 
 def quant_perblock_channel(x: torch.Tensor, block: int) -> Tuple[torch.Tensor, torch.Tensor]:

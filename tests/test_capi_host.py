@@ -48,6 +48,51 @@ def test_ctypes_struct_matches_c_layout():
     assert int(got["sizeof"]) == ctypes.sizeof(_capi.FwdParams)
 
 
+def test_append_struct_matches_c_layout():
+    fields = [f[0] for f in _capi.AppendParams._fields_]
+    body = "".join(f'printf("{f} %zu\\n", offsetof(intfa_append_params, {f}));\n' for f in fields)
+    src = f'#include <stdio.h>\n#include <stddef.h>\n#include "intfa.h"\nint main(void){{\n{body}printf("sizeof %zu\\n", sizeof(intfa_append_params));return 0;}}\n'
+    with tempfile.TemporaryDirectory() as td:
+        c = os.path.join(td, "layout.c"); exe = os.path.join(td, "layout")
+        open(c, "w").write(src)
+        subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), c, "-o", exe], check=True)
+        out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
+    got = dict(line.split() for line in out.strip().splitlines())
+    for f in fields:
+        assert int(got[f]) == getattr(_capi.AppendParams, f).offset, f
+    assert int(got["sizeof"]) == ctypes.sizeof(_capi.AppendParams)
+
+
+def test_append_validation_rejects_bad_blocks_before_touching_the_gpu():
+    lib = _capi.load()
+
+    def block(**kw):
+        a = _capi.AppendParams()
+        for n in ("k_new", "v_new", "k_cache", "v_cache", "k_scale_cache", "v_scale", "seqlens_k"):
+            setattr(a, n, 0x10000)
+        a.batch, a.heads_kv, a.seqlen_new, a.seqlen_cache, a.head_dim, a.dtype = 2, 3, 4, 64, 32, _capi.INTFA_F16
+        for t in ("kn", "vn"):
+            setattr(a, f"{t}_stride_b", 3 * 4 * 32); setattr(a, f"{t}_stride_h", 4 * 32); setattr(a, f"{t}_stride_n", 32)
+        for t in ("kc", "vc"):
+            setattr(a, f"{t}_stride_b", 3 * 64 * 32); setattr(a, f"{t}_stride_h", 64 * 32); setattr(a, f"{t}_stride_n", 32)
+        a.ksc_stride_b, a.ksc_stride_h, a.ksc_stride_n = 3 * 64, 64, 1
+        a.vs_stride_b, a.vs_stride_h = 3, 1
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+    rc = lambda **kw: lib.intfa_kvcache_append_int8(ctypes.byref(block(**kw)), None)
+    assert lib.intfa_kvcache_append_int8(None, None) == -1
+    assert rc(k_new=None) == -1 and rc(k_cache=None) == -1 and rc(k_scale_cache=None) == -1
+    assert rc(v_cache=None) == -1 and rc(v_scale=None) == -1            # v_new given: its cache and scale are required
+    assert rc(batch=0) == -7 and rc(heads_kv=0) == -7
+    assert rc(seqlen_new=0) == -3 and rc(seqlen_cache=0) == -3
+    assert rc(seqlens_k=None, seqlen_filled=65) == -3 and rc(seqlens_k=None, seqlen_filled=-1) == -3
+    assert rc(head_dim=48) == -2 and rc(dtype=_capi.INTFA_F32) == -5
+    assert rc(k_new=0x10008) == -4 and rc(kn_stride_n=36) == -4 and rc(k_cache=0x10004) == -4 and rc(vc_stride_h=12) == -4
+    assert rc(seqlens_k=0x10002) == -4
+    assert rc(kn_stride_n=16) == -7 and rc(vc_stride_n=16) == -7
+
+
 def _valid_block():
     """A parameter block that passes validation (pointers are fake but aligned; it is never launched)."""
     p = _capi.FwdParams()

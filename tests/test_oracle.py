@@ -449,3 +449,48 @@ def test_causal_with_fewer_keys_than_queries_leaves_the_first_rows_empty():
     keep = (torch.arange(100)[:, None] - 70) >= torch.arange(nk)[None, :]
     want = torch.softmax(p.masked_fill(~keep, float("-inf"))[:, :, 70:], dim=-1) @ v[:, :, :nk].float()
     assert (o[:, :, 70:].float() - want).abs().max().item() < 2e-3
+
+
+# ------------------------------------------------------------------------------------------ appending to an int8 cache
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_kvcache_append_equals_quantising_the_concatenation(dtype):
+    """K rows are quantised independently, so a cache filled by two appends must equal quant_pertoken of the concatenation
+    bit for bit (values and scales); V with the concatenation's per-(batch, head) scale must equal quant_pertensor's rows.
+    Entries are filled to different lengths; rows outside the appended ranges stay as they were."""
+    torch.manual_seed(41)
+    Z, H, d, n_cache = 2, 3, 32, 40
+    first, second = 7, 5
+    k = torch.randn((Z, H, first + second, d)).to(dtype); v = torch.randn((Z, H, first + second, d)).to(dtype)
+    k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    kc = torch.full((Z, H, n_cache, d), 99, dtype=torch.int8); vc = torch.full((Z, H, n_cache, d), 99, dtype=torch.int8)
+    ksc = torch.full((Z, H, n_cache), -1.0, dtype=dtype)
+    start = [0, 11]
+    O.kvcache_append(kc, ksc, k[:, :, :first], start, vc, vs, v[:, :, :first])
+    O.kvcache_append(kc, ksc, k[:, :, first:], [s + first for s in start], vc, vs, v[:, :, first:])
+    # (in bf16 the quotient of the largest element can round up to 128, which the harness's quantiser wraps to -128,
+    # benchmark.py:106; the append saturates such elements instead: they are compared apart)
+    over = torch.round(v / vs[:, :, None, None]).abs() > 127
+    assert dtype == torch.bfloat16 or not over.any()
+    for b in range(Z):
+        r = slice(start[b], start[b] + first + second)
+        assert torch.equal(kc[b, :, r], k8[b]) and torch.equal(ksc[b, :, r], ks[b])
+        assert torch.equal(vc[b, :, r][~over[b]], v8[b][~over[b]]) and (vc[b, :, r][over[b]].abs() == 127).all()
+        keep = torch.ones(n_cache, dtype=torch.bool); keep[r] = False
+        assert (kc[b][:, keep] == 99).all() and (vc[b][:, keep] == 99).all() and (ksc[b][:, keep] == -1).all()
+
+
+def test_kvcache_append_saturates_v_and_drops_rows_past_the_end():
+    Z, H, d, n_cache = 1, 1, 16, 4
+    kc = torch.zeros((Z, H, n_cache, d), dtype=torch.int8); vc = torch.zeros_like(kc)
+    ksc = torch.zeros((Z, H, n_cache), dtype=torch.float16)
+    k_new = torch.arange(3 * d, dtype=torch.float32).reshape(1, 1, 3, d).half() - 20
+    v_new = torch.tensor([[-1000.0, -2.0, -0.26, 0.0, 0.24, 0.26, 1.0, 126.9, 127.4, 500.0] + [0.0] * 6] * 3).reshape(1, 1, 3, d).half()
+    vs = torch.tensor([[1.0]], dtype=torch.float16)
+    O.kvcache_append(kc, ksc, k_new, [2], vc, vs, v_new)                        # room for two of the three rows
+    assert vc[0, 0, 2, :10].tolist() == [-127, -2, 0, 0, 0, 0, 1, 127, 127, 127]  # round-half-even, saturated
+    assert torch.equal(vc[0, 0, 3], vc[0, 0, 2]) and (vc[0, 0, :2] == 0).all()
+    want8, wants = O.quant_pertoken(k_new)
+    assert torch.equal(kc[0, 0, 2:], want8[0, 0, :2]) and torch.equal(ksc[0, 0, 2:], wants[0, 0, :2]) and (kc[0, 0, :2] == 0).all()
+    zs = torch.zeros((1, 1), dtype=torch.float16)
+    O.kvcache_append(kc, ksc, k_new[:, :, :1], [0], vc, zs, torch.zeros((1, 1, 1, d)).half())   # 0 / 0 -> 0
+    assert (vc[0, 0, 0] == 0).all()
