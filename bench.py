@@ -47,6 +47,8 @@ WORKLOADS = {
     "quant_pertoken_B4_H32_N4096_d128": dict(variant="quant_token", B=4, H=32, N=4096, D=128, causal=False, splits=1),
     "quant_pertensor_B4_H32_N4096_d128": dict(variant="quant_tensor", B=4, H=32, N=4096, D=128, causal=False, splits=1),
     "quant_perblock_channel_B4_H32_N4096_d128": dict(variant="quant_block", B=4, H=32, N=4096, D=128, causal=False, splits=1),
+    # new keys and values of a whole prompt quantised into an empty int8 cache (the append of a prefill)
+    "kvcache_append_B4_H32_N4096_d128": dict(variant="quant_append", B=4, H=32, N=4096, D=128, causal=False, splits=1),
 }
 # HBM bytes per launch of the forward kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
 # what the same counter reads for a plain copy of known size; None where not measured.
@@ -108,12 +110,20 @@ def bench_quant(args, variant, x, B, H, N, D, dt):
     reads its input twice (maximum, then quantise)."""
     import torch
     import int_flashattention_amd as M
-    fn = {"quant_token": M.quant_pertoken, "quant_tensor": M.quant_pertensor,
-          "quant_block": lambda t: M.quant_perblock_channel(t, 128)}[variant]
+    if variant == "quant_append":          # K and V of the prompt into an empty cache: reads both inputs once, writes both caches
+        kc = torch.zeros((B, H, N, D), dtype=torch.int8, device=x.device); vc = torch.zeros_like(kc)
+        ksc = torch.zeros((B, H, N), dtype=x.dtype, device=x.device)
+        vs = (x.abs().amax(dim=(2, 3)) / 127).to(x.dtype)
+        v_new = x.flip(2).contiguous()
+        fn = lambda t: M.kvcache_append(kc, ksc, t, 0, vc, vs, v_new)
+    else:
+        fn = {"quant_token": M.quant_pertoken, "quant_tensor": M.quant_pertensor,
+              "quant_block": lambda t: M.quant_perblock_channel(t, 128)}[variant]
     n = B * H * N * D
     # (the per-block variant reads its block twice too, but the second sweep of 32 KiB is served by the cache)
-    scale_bytes = {"quant_token": 2 * B * H * N, "quant_tensor": 2 * B * H, "quant_block": 4 * B * H * (N // 128) * D}[variant]
-    alg_bytes = (2 + 1) * n + scale_bytes + (2 * n if variant == "quant_tensor" else 0)
+    scale_bytes = {"quant_token": 2 * B * H * N, "quant_tensor": 2 * B * H, "quant_block": 4 * B * H * (N // 128) * D,
+                   "quant_append": 2 * B * H * N + 2 * B * H}[variant]
+    alg_bytes = (2 + 1) * n * (2 if variant == "quant_append" else 1) + scale_bytes + (2 * n if variant == "quant_tensor" else 0)
     for _ in range(args.warmup):
         fn(x)
     torch.cuda.synchronize()
@@ -132,7 +142,8 @@ def bench_quant(args, variant, x, B, H, N, D, dt):
            "roofline": {"bound": "hbm", "achieved": alg_bytes / (kern_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": alg_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
                         "kernel": {"quant_token": "quant_pertoken_kernel", "quant_block": "quant_blockchan_kernel",
-                                   "quant_tensor": "quant_slice_amax_kernel + quant_slice_apply_kernel"}[variant],
+                                   "quant_tensor": "quant_slice_amax_kernel + quant_slice_apply_kernel",
+                                   "quant_append": "kv_append_kernel (keys) + kv_append_kernel (values)"}[variant],
                         "avg_launch_ms": kern_ms}}
     print(json.dumps(out))
 

@@ -309,53 +309,66 @@ struct AppendParams {
 
 template <int DT, int LPR, bool IS_V> __global__ void __launch_bounds__(256) kv_append_kernel(const AppendParams p) {
     constexpr int RPB = 256 / LPR;
+    constexpr int U = 4;                          // rows a lane has in flight
     const AppendSide& s = IS_V ? p.v : p.k;
     const int sub = threadIdx.x % LPR, rl = threadIdx.x / LPR;
     const uint32_t step = gridDim.x * RPB, rows = (uint32_t)p.rows;
-    // (the trip count depends on the workgroup only through rl, and rows is a multiple of nothing: the lanes of a row
-    // share rl, so they enter and leave the loop together and the shuffles below see all of them)
-    for (uint32_t row = blockIdx.x * RPB + rl; row < rows; row += step) {
-        const uint32_t bh = row / (uint32_t)p.seqlen_new, i = row - bh * (uint32_t)p.seqlen_new;
-        const uint32_t b = bh / (uint32_t)p.heads, h = bh - b * (uint32_t)p.heads;
-        int len = p.seqlen_filled;
-        if (p.seqlens_k != nullptr) {
-            const int n = p.seqlens_k[b];
-            len = n < 0 ? 0 : (n < p.seqlen_cache ? n : p.seqlen_cache);
+    // (the lanes of a row share rl, so they enter and leave the loop together and the shuffles below see all of them)
+    for (uint32_t row0 = blockIdx.x * RPB + rl; row0 < rows; row0 += step * U) {
+        v4i raw[U];
+        uint32_t bq[U], hq[U], iq[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t row = row0 + u * step;
+            const uint32_t bh = row / (uint32_t)p.seqlen_new;
+            iq[u] = row - bh * (uint32_t)p.seqlen_new;
+            bq[u] = bh / (uint32_t)p.heads; hq[u] = bh - bq[u] * (uint32_t)p.heads;
+            raw[u] = row < rows ? *(const v4i*)(s.x + bq[u] * s.xb + hq[u] * s.xh + iq[u] * s.xn + sub * 16) : (v4i){0, 0, 0, 0};
         }
-        const int64_t pos = (int64_t)len + i;
-        const v4i raw = *(const v4i*)(s.x + b * s.xb + h * s.xh + i * s.xn + sub * 16);
-        uint16_t sbits;
-        if (IS_V) {
-            sbits = ((const uint16_t*)s.scale)[b * s.sb + h * s.sh];
-        } else {
-            uint32_t m = amax8(raw);
 #pragma unroll
-            for (int off = LPR / 2; off > 0; off >>= 1) {
-                const uint32_t o = (uint32_t)__shfl_xor((int)m, off, 64);
-                m = m > o ? m : o;
-            }
-            sbits = from_f32<DT>(to_f32<DT>((uint16_t)m) / 127.0f);
-        }
-        if (pos >= p.seqlen_cache) continue;                                   // no room: the row is dropped
-        char* dst = s.cache + b * s.cb + h * s.ch + pos * s.cn + sub * 8;
-        const RowDivisor d = make_divisor(to_f32<DT>(sbits));
-        if (IS_V) {
-            int out[2];
+        for (int u = 0; u < U; ++u) {
+            const uint32_t row = row0 + u * step;
+            const uint32_t b = bq[u], h = hq[u];
+            uint16_t sbits = 0;
+            if (IS_V) {
+                if (row < rows) sbits = ((const uint16_t*)s.scale)[b * s.sb + h * s.sh];
+            } else {
+                uint32_t m = amax8(raw[u]);
 #pragma unroll
-            for (int w = 0; w < 2; ++w) {
-                float q[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t word = (uint32_t)raw[2 * w + j / 2];
-                    const float t = quotient16<DT>((uint16_t)(j & 1 ? word >> 16 : word & 0xffffu), d);
-                    q[j] = t != t ? t : __builtin_fminf(__builtin_fmaxf(t, -127.0f), 127.0f);      // (NaN from 0 / 0 stays NaN: byte 0)
+                for (int off = LPR / 2; off > 0; off >>= 1) {
+                    const uint32_t o = (uint32_t)__shfl_xor((int)m, off, 64);
+                    m = m > o ? m : o;
                 }
-                out[w] = (int)pack4_rne(q[0], q[1], q[2], q[3]);
+                sbits = from_f32<DT>(to_f32<DT>((uint16_t)m) / 127.0f);
             }
-            *(v2i*)dst = (v2i){out[0], out[1]};
-        } else {
-            if (sub == 0) ((uint16_t*)s.scale)[b * s.sb + h * s.sh + pos * s.sn] = sbits;
-            quant_store8<DT>(raw, d, dst);
+            if (row >= rows) continue;
+            int len = p.seqlen_filled;
+            if (p.seqlens_k != nullptr) {
+                const int n = p.seqlens_k[b];
+                len = n < 0 ? 0 : (n < p.seqlen_cache ? n : p.seqlen_cache);
+            }
+            const int64_t pos = (int64_t)len + iq[u];
+            if (pos >= p.seqlen_cache) continue;                               // no room: the row is dropped
+            char* dst = s.cache + b * s.cb + h * s.ch + pos * s.cn + sub * 8;
+            const RowDivisor d = make_divisor(to_f32<DT>(sbits));
+            if (IS_V) {
+                int out[2];
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+                    float q[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t word = (uint32_t)raw[u][2 * w + j / 2];
+                        const float t = quotient16<DT>((uint16_t)(j & 1 ? word >> 16 : word & 0xffffu), d);
+                        q[j] = t != t ? t : __builtin_fminf(__builtin_fmaxf(t, -127.0f), 127.0f);  // (NaN from 0 / 0 stays NaN: byte 0)
+                    }
+                    out[w] = (int)pack4_rne(q[0], q[1], q[2], q[3]);
+                }
+                *(v2i*)dst = (v2i){out[0], out[1]};
+            } else {
+                if (sub == 0) ((uint16_t*)s.scale)[b * s.sb + h * s.sh + pos * s.sn] = sbits;
+                quant_store8<DT>(raw[u], d, dst);
+            }
         }
     }
 }
