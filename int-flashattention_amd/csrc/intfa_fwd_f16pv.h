@@ -37,8 +37,10 @@ template <int D> struct F16PvGeom {
     static constexpr int NHALF = D / DV;
 };
 
+// (16-bit K tiles at head_dim 256 are 32 KiB each: double-buffered beside the V tiles they leave room for one workgroup
+// per compute unit, whatever the register count)
 template <bool QK_INT8, int D, bool CAUSAL, int IO_DT, bool SPLIT>
-__global__ void __launch_bounds__(kThreads, 2) fwd_f16pv_kernel(const KParams p) {
+__global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f16pv_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr int BN = kBlockN16, NST = BN / 32;
     constexpr int QB = QK_INT8 ? 1 : 2;               // bytes per Q/K element
