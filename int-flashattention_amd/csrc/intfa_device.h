@@ -185,7 +185,10 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // operations: fp16(p) (round to nearest even) * 127 -> fp16, + 0.5 -> fp16, truncating conversion to an integer.  The
 // multiply and the add are the packed fp16 instructions (two values each; kept apart: a fused multiply-add would skip
 // the rounding of the product); the two conversions write their byte straight into the packed word (SDWA destination
-// select), bytes B0 and B0 + 1 of pk.  B0 = 0 starts a new word.
+// select), bytes B0 and B0 + 1 of pk.  B0 = 0 starts a new word.  A write with a destination select needs one wait
+// state before the next vector instruction reads that register (the following conversion does, to preserve the other
+// bytes, and so does the MFMA that takes the finished word); the compiler places such wait states for its own
+// instructions only, hence the s_nop behind each conversion.
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 template <int B0> __device__ __forceinline__ unsigned requant_p_reference2(float p0, float p1, unsigned pk) {
     static_assert(B0 == 0 || B0 == 2, "two byte pairs per word");
@@ -197,11 +200,11 @@ template <int B0> __device__ __forceinline__ unsigned requant_p_reference2(float
     }
     const unsigned hb = __builtin_bit_cast(unsigned, h);
     if (B0 == 0) {
-        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:WORD_0" : "=v"(pk) : "v"(hb));
-        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1" : "+v"(pk) : "v"(hb));
+        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:WORD_0\n\ts_nop 0" : "=v"(pk) : "v"(hb));
+        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\ts_nop 0" : "+v"(pk) : "v"(hb));
     } else {
-        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0" : "+v"(pk) : "v"(hb));
-        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1" : "+v"(pk) : "v"(hb));
+        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0\n\ts_nop 0" : "+v"(pk) : "v"(hb));
+        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\ts_nop 0" : "+v"(pk) : "v"(hb));
     }
     return pk;
 }

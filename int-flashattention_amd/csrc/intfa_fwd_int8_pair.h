@@ -6,8 +6,8 @@
 // waves w and w + 4 (same SIMD) share the query rows 32w .. 32w+31:
 //   * wave w + 4h computes S^T, the scaling, the row maxima, the exponentials and the int8 P of the keys 32h .. 32h+31
 //     of the block (one 32-key sub-tile each);
-//   * the two exchange their row maxima and their packed P fragments through LDS (two workgroup barriers per block on
-//     top of the one that publishes the K/V tiles);
+//   * the two exchange their row maxima and their packed P fragments through LDS (the block's two workgroup barriers,
+//     which also publish the V tile and the next block's K tile);
 //   * wave w + 4h multiplies the whole P (64 keys) with the columns 128h .. 128h+127 of V and owns those output
 //     columns; the row sum is kept per wave and added up in the epilogue.
 // No vector instruction is issued twice for the same element.  Waves 0-3 copy the K tile of the next block, waves 4-7
