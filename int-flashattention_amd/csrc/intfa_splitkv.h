@@ -18,10 +18,14 @@ __global__ void __launch_bounds__(256) splitkv_combine_kernel(const KParams p) {
     // log-sum-exp over splits (every lane of a row computes the same scalars)
     float lse_max = -INFINITY;
     for (int s = 0; s < ns; ++s) lse_max = fmaxf(lse_max, p.lse_part[(int64_t)s * rows + row]);
-    if (lse_max == -INFINITY) lse_max = 0.f;
+    // A row no split saw a key for (an empty cache entry, a causal row above the first key): every partial is -inf and
+    // the result is zeros with lse = -inf, the value the single-pass kernels write for such a row - the neutral element
+    // for a caller that merges results by lse.
+    const bool empty = lse_max == -INFINITY;
+    if (empty) lse_max = 0.f;
     float sum = 0.f;
     for (int s = 0; s < ns; ++s) sum += fast_exp2(p.lse_part[(int64_t)s * rows + row] - lse_max);
-    const float lse = (sum == 0.f || sum != sum) ? INFINITY : __builtin_log2f(sum) + lse_max;
+    const float lse = empty ? -INFINITY : __builtin_log2f(sum) + lse_max;     // (a NaN partial propagates as NaN)
     v4f acc = {0.f, 0.f, 0.f, 0.f};
     const float* op0 = p.o_part + row * D + sub * 4;
     const int64_t sstride = rows * D;
@@ -32,7 +36,7 @@ __global__ void __launch_bounds__(256) splitkv_combine_kernel(const KParams p) {
         for (int u = 0; u < 4; ++u) {
             const int s = s0 + u < ns ? s0 + u : ns - 1;                 // clamped loads, zero weight past the end
             part[u] = *(const v4f*)(op0 + (int64_t)s * sstride);
-            w[u] = s0 + u < ns ? fast_exp2(p.lse_part[(int64_t)s * rows + row] - lse) : 0.f;
+            w[u] = (s0 + u < ns && !empty) ? fast_exp2(p.lse_part[(int64_t)s * rows + row] - lse) : 0.f;
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u)

@@ -340,10 +340,14 @@ def splitkv_combine(o_parts: torch.Tensor, lse_parts: torch.Tensor) -> Tuple[tor
     are m + log2(l), -inf for a split that saw no key.
     """
     lse_max = lse_parts.max(dim=0).values
-    lse_max = torch.where(torch.isinf(lse_max), torch.zeros_like(lse_max), lse_max)
+    empty = torch.isinf(lse_max) & (lse_max < 0)            # no split saw a key for this row
+    lse_max = torch.where(empty, torch.zeros_like(lse_max), lse_max)
     lse_sum = torch.exp2(lse_parts - lse_max).sum(dim=0)
-    lse = torch.where(lse_sum == 0, torch.full_like(lse_sum, float("inf")), torch.log2(lse_sum) + lse_max)
-    w = torch.exp2(lse_parts - lse)
+    # the weights of an empty row are zero (the reference gets there by setting the row's lse to +inf, :1226); the lse
+    # REPORTED for such a row is -inf, as for a single pass over no key (the neutral element of a merge by lse)
+    lse_w = torch.where(empty, torch.full_like(lse_sum, float("inf")), torch.log2(lse_sum) + lse_max)
+    w = torch.exp2(lse_parts - lse_w)
+    lse = torch.where(empty, torch.full_like(lse_sum, float("-inf")), lse_w)
     return (w[..., None] * o_parts).sum(dim=0), lse
 
 

@@ -206,7 +206,7 @@ def test_causal_decode_matches_oracle(B, H, H_kv, Nq, Nk, D, p_round):
     assert torch.isfinite(o).all()
     empty = max(Nq - Nk, 0)
     if empty:
-        assert o[:, :, :empty].abs().max().item() == 0 and torch.isinf(lse[:, :, :empty]).all()
+        assert o[:, :, :empty].abs().max().item() == 0 and torch.isinf(lse[:, :, :empty]).all() and (lse[:, :, :empty] < 0).all()
     assert max_abs(o, ref) <= MAX_ABS and mean_rel(o, ref) <= 2e-3
     assert (lse.cpu()[:, :, empty:] - lse_ref[:, :, empty:]).abs().max().item() < 1e-3
     if Nq == 1:

@@ -484,7 +484,7 @@ def test_causal_with_separate_lengths_is_aligned_bottom_right(variant, Nq, Nk, D
     assert torch.isfinite(o).all()
     empty = max(Nq - Nk, 0)
     if empty:
-        assert o[:, :, :empty].abs().max().item() == 0 and torch.isinf(lse[:, :, :empty]).all()
+        assert o[:, :, :empty].abs().max().item() == 0 and torch.isinf(lse[:, :, :empty]).all() and (lse[:, :, :empty] < 0).all()
     assert (lse.cpu()[:, :, empty:] - lse_ref[:, :, empty:]).abs().max().item() < 2e-3
 
 
@@ -513,6 +513,39 @@ def test_causal_separate_lengths_with_split_kv_and_per_batch_lengths(variant):
         ref = one(b, n)
         assert max_abs(o[b:b + 1], ref) <= 4e-3, (b, n)
         assert max_abs(o3[b:b + 1], ref) <= MAX_ABS and mean_rel(o3[b:b + 1], ref) <= 3e-2, (b, n)
+
+
+@pytest.mark.parametrize("num_splits", [2, 4, "auto"])
+@pytest.mark.parametrize("Nq", [2, 150])            # the decode-shaped kernel and the general one
+def test_rows_without_a_key_on_the_split_path_give_zeros_and_minus_inf_lse(num_splits, Nq):
+    """A batch entry whose cache is empty and (causal, fewer keys than queries) the rows above the first key: zeros and
+    lse = -inf whether the call runs as one pass or as split partials merged by the combine kernel."""
+    B, H, Nk, D = 3, 2, 1200, 128
+    g = torch.Generator().manual_seed(47)
+    q = torch.randn((B, H, Nq, D), generator=g).half()
+    k = torch.randn((B, H, Nk, D), generator=g).half()
+    v = torch.randn((B, H, Nk, D), generator=g).half()
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
+    sm = D ** -0.5
+    lens = [1200, 0, 77]
+    sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    for causal in (False, True):
+        o, lse = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), causal, sm, seqlens_k=sl, num_splits=num_splits,
+                                       return_lse=True)
+        o1, lse1 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), causal, sm, seqlens_k=sl, return_lse=True)
+        torch.cuda.synchronize()
+        assert torch.isfinite(o).all()
+        assert o[1].abs().max().item() == 0 and torch.isinf(lse[1]).all() and (lse[1] < 0).all()
+        if causal:                                     # entry 2 has 77 keys: rows 0 .. Nq - 78 see none of them
+            empty = max(Nq - lens[2], 0)
+            if empty:
+                assert o[2, :, :empty].abs().max().item() == 0
+                assert torch.isinf(lse[2, :, :empty]).all() and (lse[2, :, :empty] < 0).all()
+            assert torch.isfinite(lse[2, :, empty:]).all()
+        # the sign and the finite values agree with the single pass (the split frames differ in P8 only)
+        assert torch.equal(torch.isinf(lse), torch.isinf(lse1)) and torch.equal(lse < 0, lse1 < 0)
+        fin = torch.isfinite(lse1)
+        assert (lse[fin] - lse1[fin]).abs().max().item() < 1e-3
 
 
 # ------------------------------------------------------------------------------------------ grouped K/V heads

@@ -444,7 +444,7 @@ def test_causal_with_fewer_keys_than_queries_leaves_the_first_rows_empty():
     q, k, v, _ = O.make_inputs(1, 1, 100, 16, seed=19)
     nk = 30                                                                      # row i sees keys 0 .. i - 70
     o, lse = O.attention_fp(q, k[:, :, :nk], v[:, :, :nk], True, 0.3, block_m=64, block_n=64, return_lse=True)
-    assert o[:, :, :70].abs().max().item() == 0 and torch.isinf(lse[:, :, :70]).all()
+    assert o[:, :, :70].abs().max().item() == 0 and torch.isinf(lse[:, :, :70]).all() and (lse[:, :, :70] < 0).all()
     p = (q.float() @ k[:, :, :nk].float().transpose(2, 3)) * 0.3
     keep = (torch.arange(100)[:, None] - 70) >= torch.arange(nk)[None, :]
     want = torch.softmax(p.masked_fill(~keep, float("-inf"))[:, :, 70:], dim=-1) @ v[:, :, :nk].float()
