@@ -20,6 +20,37 @@ sys.path.insert(0, ROOT)
 INT8_PEAK_TOPS = 5033.0      # MI355X dense int8 MFMA: 256 CUs x 2.4 GHz x 8192 ops/clk/CU
 FP16_PEAK_TFLOPS = 2516.6
 HBM_PEAK_GBS = 8000.0
+INT8_OPS_PER_CLK_CU = 8192   # v_mfma_i32_32x32x32_i8: 65536 ops in 8 passes of 4 clocks on each of a CU's 4 SIMDs
+FP16_FLOPS_PER_CLK_CU = 4096
+
+
+def device_peak_check(torch, dev):
+    """The peak recomputed from what the device reports (compute units x maximum engine clock x ops per clock and CU: the
+    first GPU agent of `rocminfo`, the compute-unit count also from the runtime), printed beside the datasheet constants
+    the fractions are priced against."""
+    import re
+    import subprocess
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    name, mhz, cus_rocminfo = torch.cuda.get_device_properties(dev).name, None, None
+    try:
+        txt = subprocess.run(["/opt/rocm/bin/rocminfo"], capture_output=True, text=True, timeout=30).stdout
+        for agent in txt.split("*******")[1:]:
+            if re.search(r"Device Type:\s+GPU", agent):
+                m = re.search(r"Max Clock Freq\. \(MHz\):\s+(\d+)", agent)
+                c = re.search(r"Compute Unit:\s+(\d+)", agent)
+                mhz = float(m.group(1)) if m else None
+                cus_rocminfo = int(c.group(1)) if c else None
+                break
+    except Exception as e:          # rocminfo missing or unreadable: report what the runtime alone gives
+        name += f" (rocminfo unavailable: {type(e).__name__})"
+    out = {"device": name, "compute_units": cus, "compute_units_rocminfo": cus_rocminfo, "max_engine_clock_mhz": mhz,
+           "int8_ops_per_clk_cu": INT8_OPS_PER_CLK_CU, "fp16_flops_per_clk_cu": FP16_FLOPS_PER_CLK_CU,
+           "priced_against": {"int8_tops": INT8_PEAK_TOPS, "fp16_tflops": FP16_PEAK_TFLOPS, "hbm_gbs": HBM_PEAK_GBS}}
+    if mhz:
+        out["int8_tops"] = cus * mhz * 1e6 * INT8_OPS_PER_CLK_CU / 1e12
+        out["fp16_tflops"] = cus * mhz * 1e6 * FP16_FLOPS_PER_CLK_CU / 1e12
+    return out
+
 
 # name: variant, B, H, N, D, causal, num_splits, input dtype, std of Q/K/V, fraction of K channels multiplied by 20
 WORKLOADS = {
@@ -50,14 +81,20 @@ WORKLOADS = {
     # new keys and values of a whole prompt quantised into an empty int8 cache (the append of a prefill)
     "kvcache_append_B4_H32_N4096_d128": dict(variant="quant_append", B=4, H=32, N=4096, D=128, causal=False, splits=1),
 }
-# HBM bytes per launch of the forward kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
-# what the same counter reads for a plain copy of known size; None where not measured.
+# HBM bytes per launch of the forward kernel as measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
+# what the same counter reads for a plain copy of known size.  These are constants taken from the profile named beside
+# them, NOT measured in the run that prints them (counters need the profiler); workloads without a profile report None.
 MEASURED_TRAFFIC_BYTES = {
     # FETCH_SIZE x 1.9997 + WRITE_SIZE x 1.0 (KiB per dispatch, factors from a 256 MiB copy): 194.2 MiB read + 128 MiB written
-    "full_int8_B4_H32_N4096_d128": 337902723,
+    "full_int8_B4_H32_N4096_d128": (337902723, "profiles/fwd_full_int8_d128_B4_H32_N4096.txt"),
     # FETCH_SIZE 528548.6 x 1.9998 + WRITE_SIZE 256 x 1.0: 1032.2 MiB read + 0.25 MiB written (algorithmic: 1082523648)
-    "full_int8_decode_B32_H32_Nq1_Nk4096_d128": 1082605181,
+    "full_int8_decode_B32_H32_Nq1_Nk4096_d128": (1082605181, "profiles/fwd_decode_full_int8_d128_B32_H32_Nq1_Nk4096.txt"),
 }
+
+
+def traffic_of(workload):
+    t = MEASURED_TRAFFIC_BYTES.get(workload)
+    return (t[0], f"constant from {t[1]} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)") if t else (None, None)
 
 
 def ops_of(B, H, N, D, causal):
@@ -133,7 +170,8 @@ def bench_quant(args, variant, x, B, H, N, D, dt):
         e0.record(); fn(x); e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    kern_ms = statistics.fmean(e0.elapsed_time(e1) for e0, e1 in evs)
+    per_launch_ms = [e0.elapsed_time(e1) for e0, e1 in evs]
+    kern_ms = statistics.fmean(per_launch_ms)
     ms_step = wall * 1e3 / args.steps
     out = {"metric": "input quantiser throughput (algorithmic HBM bytes per second)", "value": alg_bytes / (ms_step * 1e-3) / 1e9,
            "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
@@ -144,7 +182,8 @@ def bench_quant(args, variant, x, B, H, N, D, dt):
                         "kernel": {"quant_token": "quant_pertoken_kernel", "quant_block": "quant_blockchan_kernel",
                                    "quant_tensor": "quant_slice_amax_kernel + quant_slice_apply_kernel",
                                    "quant_append": "kv_append_kernel (keys) + kv_append_kernel (values)"}[variant],
-                        "avg_launch_ms": kern_ms}}
+                        "avg_launch_ms": kern_ms, "median_launch_ms": statistics.median(per_launch_ms)},
+           "peak_check": device_peak_check(torch, x.device)}
     print(json.dumps(out))
 
 
@@ -157,6 +196,8 @@ def main():
     ap.add_argument("--p-round", default="rne", choices=["rne", "reference"])
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU-baseline budget; 0 skips it")
     ap.add_argument("--no-parity", action="store_true", help="skip the oracle check of one head")
+    ap.add_argument("--no-other-rounding", action="store_true",
+                    help="full-int8: do not also time the workload in the other rounding of P")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run one device-to-device copy of this many MiB before the timed region: a kernel of known "
                          "HBM traffic that calibrates FETCH_SIZE / WRITE_SIZE when the run is under rocprofv3 --pmc")
@@ -221,8 +262,25 @@ def main():
     per_launch_ms = [e0.elapsed_time(e1) for e0, e1 in evs]
     ms_step = wall * 1e3 / args.steps
     kern_ms = statistics.fmean(per_launch_ms)
+    kern_med_ms = statistics.median(per_launch_ms)
     value = ops / (ms_step * 1e-3) / 1e12
     achieved = ops / (kern_ms * 1e-3) / 1e12
+
+    # the same workload in the other rounding of P (full-int8 only), per-launch HIP events as above
+    other_round = None
+    if variant == "full" and not args.no_other_rounding:
+        other = "reference" if args.p_round == "rne" else "rne"
+        step_o = lambda: M.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, out_dtype=dt, num_splits=splits,
+                                               p_round=other, v_scale_block=v_block)
+        for _ in range(max(3, args.warmup // 5)):
+            step_o()
+        torch.cuda.synchronize()
+        evo = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for e0, e1 in evo:
+            e0.record(); step_o(); e1.record()
+        torch.cuda.synchronize()
+        mo = [e0.elapsed_time(e1) for e0, e1 in evo]
+        other_round = {"p_round": other, "avg_launch_ms": statistics.fmean(mo), "median_launch_ms": statistics.median(mo)}
 
     parity = None
     if not args.no_parity:
@@ -253,7 +311,12 @@ def main():
             refs["vs_oracle"] = O.attention_int8(c(q8), c(k8), c(v), c(qs), c(ks), causal, sm, block_n=bn, out_dtype=dt)
         else:
             refs["vs_oracle"] = O.attention_fp(c(q), c(k), c(v), causal, sm, block_n=bn)
-        err = lambda x, y: {"max_abs": (x - y).abs().max().item(), "mean_rel": ((x - y).abs().mean() / y.abs().mean()).item()}
+        # max_abs / mean_rel (= mean|x-y| / mean|y|) are the measures the tolerances are stated in; mre_reference is the
+        # reference harness's own measure (benchmark.py:110-122: mean(|y-x| / (|y| + 1e-5)), x the kernel's output), over
+        # every element of the slice and over the last four (its CALC_NUM = 4)
+        err = lambda x, y: {"max_abs": (x - y).abs().max().item(), "mean_rel": ((x - y).abs().mean() / y.abs().mean()).item(),
+                            "mre_reference": O.mean_relative_error(x, y),
+                            "mre_reference_calc_num_4": O.mean_relative_error(x, y, calc_num=4)}
         parity = {"slice": f"batch {b}, head {h}", "oracle_block_n": bn}
         for name, r in refs.items():
             parity[name] = err(got, r.float())
@@ -284,10 +347,19 @@ def main():
                                  else ", V per-(batch,head) int8") if variant == "full" else "")},
         "pct_int8_peak": 100.0 * value / INT8_PEAK_TOPS,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TOP/s" if variant == "full" else "TFLOP/s",
-                     "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "kernel": kernel_name, "avg_launch_ms": kern_ms, "peak_model": peak_model,
+                     "frac": achieved / peak, "traffic": traffic_of(args.workload)[0], "traffic_source": traffic_of(args.workload)[1],
+                     "kernel": kernel_name, "avg_launch_ms": kern_ms, "median_launch_ms": kern_med_ms,
+                     "achieved_at_median": ops / (kern_med_ms * 1e-3) / 1e12, "peak_model": peak_model,
                      "launch_includes": "forward kernel" + (" + split-KV combine kernel" if splits != 1 else "")},
+        "peak_check": device_peak_check(torch, dev),
     }
+    if other_round is not None:
+        a_o = ops / (other_round["avg_launch_ms"] * 1e-3) / 1e12
+        out["roofline_" + other_round["p_round"] + "_rounding"] = {
+            "bound": "mfma", "achieved": a_o, "peak": peak, "unit": "TOP/s", "frac": a_o / peak, "kernel": kernel_name,
+            "p_round": other_round["p_round"], "avg_launch_ms": other_round["avg_launch_ms"],
+            "median_launch_ms": other_round["median_launch_ms"],
+            "slowdown_vs_timed_rounding": other_round["avg_launch_ms"] / kern_ms}
     if decode:
         # one pass over the cached K and V (int8) and their scales; Q, O and the split partials are a rounding error
         sb = 2 if dt != torch.float32 else 4
@@ -299,8 +371,8 @@ def main():
         out["config"]["bytes_per_step"] = alg_bytes
         out.pop("pct_int8_peak")
         out["roofline"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                           "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "kernel": "fwd_decode_full_int8_kernel",
-                           "avg_launch_ms": kern_ms,
+                           "traffic": traffic_of(args.workload)[0], "traffic_source": traffic_of(args.workload)[1],
+                           "kernel": "fwd_decode_full_int8_kernel", "avg_launch_ms": kern_ms, "median_launch_ms": kern_med_ms,
                            "launch_includes": "forward kernel" + (" + split-KV combine kernel" if splits != 1 else "")}
     if parity is not None:
         out["parity"] = parity

@@ -191,32 +191,52 @@ __device__ __forceinline__ float half_pair_sum(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// The reference's requantisation of P (flash_atten_full_int8.py:49-51) for two probabilities at once, in its own fp16
-// operations: fp16(p) (round to nearest even) * 127 -> fp16, + 0.5 -> fp16, truncating conversion to an integer.  The
-// multiply and the add are the packed fp16 instructions (two values each; kept apart: a fused multiply-add would skip
-// the rounding of the product); the two conversions write their byte straight into the packed word (SDWA destination
-// select), bytes B0 and B0 + 1 of pk.  B0 = 0 starts a new word.  A write with a destination select needs one wait
-// state before the next vector instruction reads that register (the following conversion does, to preserve the other
-// bytes, and so does the MFMA that takes the finished word); the compiler places such wait states for its own
-// instructions only, hence the s_nop behind each conversion.
+// The reference's requantisation of P (flash_atten_full_int8.py:49-51) for the 16 probabilities a lane holds of one 32-key
+// sub-tile, in the reference's own fp16 operations: fp16(p) (round to nearest even) * 127 -> fp16, + 0.5 -> fp16,
+// truncating conversion to an integer.  The multiply and the add are the packed fp16 instructions (two values each; kept
+// apart: a fused multiply-add would skip the rounding of the product).  The sixteen truncating conversions write their
+// byte straight into the four packed words (SDWA destination select).  A write with a destination select needs one wait
+// state before the next vector instruction touches that register, and the compiler places wait states for its own
+// instructions only: the conversions are therefore issued word-interleaved (bytes 0 of the four words, then bytes 1, ...),
+// so that three other conversions lie between two writes to one word, each round as ONE asm statement so that nothing can
+// be scheduled into it, and a single s_nop closes the last round before the words can be consumed.
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
-template <int B0> __device__ __forceinline__ unsigned requant_p_reference2(float p0, float p1, unsigned pk) {
-    static_assert(B0 == 0 || B0 == 2, "two byte pairs per word");
-    v2h h = {(_Float16)p0, (_Float16)p1};
-    {
+typedef float v2f __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ v4i requant_p_reference16(const float (&p)[16]) {
+    unsigned hb[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        v2h h = __builtin_convertvector((v2f){p[2 * i], p[2 * i + 1]}, v2h);
+        {
 #pragma clang fp contract(off)
-        h = h * (v2h){(_Float16)127.0f, (_Float16)127.0f};
-        h = h + (v2h){(_Float16)0.5f, (_Float16)0.5f};
+            h = h * (v2h){(_Float16)127.0f, (_Float16)127.0f};
+            h = h + (v2h){(_Float16)0.5f, (_Float16)0.5f};
+        }
+        hb[i] = __builtin_bit_cast(unsigned, h);
     }
-    const unsigned hb = __builtin_bit_cast(unsigned, h);
-    if (B0 == 0) {
-        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:WORD_0\n\ts_nop 0" : "=v"(pk) : "v"(hb));
-        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\ts_nop 0" : "+v"(pk) : "v"(hb));
-    } else {
-        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0\n\ts_nop 0" : "+v"(pk) : "v"(hb));
-        asm("v_cvt_u16_f16_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\ts_nop 0" : "+v"(pk) : "v"(hb));
-    }
-    return pk;
+    unsigned w0, w1, w2, w3;
+    asm volatile("v_cvt_u16_f16_sdwa %0, %4 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:WORD_0\n\t"
+                 "v_cvt_u16_f16_sdwa %1, %5 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:WORD_0\n\t"
+                 "v_cvt_u16_f16_sdwa %2, %6 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:WORD_0\n\t"
+                 "v_cvt_u16_f16_sdwa %3, %7 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:WORD_0"
+                 : "=&v"(w0), "=&v"(w1), "=&v"(w2), "=&v"(w3) : "v"(hb[0]), "v"(hb[2]), "v"(hb[4]), "v"(hb[6]));
+    asm volatile("v_cvt_u16_f16_sdwa %0, %4 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\t"
+                 "v_cvt_u16_f16_sdwa %1, %5 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\t"
+                 "v_cvt_u16_f16_sdwa %2, %6 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\t"
+                 "v_cvt_u16_f16_sdwa %3, %7 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1"
+                 : "+v"(w0), "+v"(w1), "+v"(w2), "+v"(w3) : "v"(hb[0]), "v"(hb[2]), "v"(hb[4]), "v"(hb[6]));
+    asm volatile("v_cvt_u16_f16_sdwa %0, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0\n\t"
+                 "v_cvt_u16_f16_sdwa %1, %5 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0\n\t"
+                 "v_cvt_u16_f16_sdwa %2, %6 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0\n\t"
+                 "v_cvt_u16_f16_sdwa %3, %7 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0"
+                 : "+v"(w0), "+v"(w1), "+v"(w2), "+v"(w3) : "v"(hb[1]), "v"(hb[3]), "v"(hb[5]), "v"(hb[7]));
+    asm volatile("v_cvt_u16_f16_sdwa %0, %4 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\t"
+                 "v_cvt_u16_f16_sdwa %1, %5 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\t"
+                 "v_cvt_u16_f16_sdwa %2, %6 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\t"
+                 "v_cvt_u16_f16_sdwa %3, %7 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\t"
+                 "s_nop 0"
+                 : "+v"(w0), "+v"(w1), "+v"(w2), "+v"(w3) : "v"(hb[1]), "v"(hb[3]), "v"(hb[5]), "v"(hb[7]));
+    return (v4i){(int)w0, (int)w1, (int)w2, (int)w3};
 }
 
 }  // namespace intfa

@@ -254,21 +254,24 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
         const float bias = (PROUND == 0 ? kLog2_127 : 0.f) - m_new;
         float lsum = 0.f;
         v4i p8;
+        {
+            float e[16];
 #pragma unroll
-        for (int w4 = 0; w4 < 4; ++w4) {
-            unsigned pk = 0;
-            float e[4];
+            for (int r = 0; r < 16; ++r) {
+                e[r] = fast_exp2(fmaf(x[r], qsc, bias));                         // RNE mode: 127 * p
+                lsum += e[r];
+            }
+            if (PROUND == 0) {
 #pragma unroll
-            for (int b4 = 0; b4 < 4; ++b4) {
-                e[b4] = fast_exp2(fmaf(x[4 * w4 + b4], qsc, bias));              // RNE mode: 127 * p
-                lsum += e[b4];
-                if (PROUND == 0) pk = __builtin_amdgcn_cvt_pk_u8_f32(e[b4], b4, pk);
+                for (int w4 = 0; w4 < 4; ++w4) {
+                    unsigned pk = 0;
+#pragma unroll
+                    for (int b4 = 0; b4 < 4; ++b4) pk = __builtin_amdgcn_cvt_pk_u8_f32(e[4 * w4 + b4], b4, pk);
+                    p8[w4] = (int)pk;
+                }
+            } else {
+                p8 = requant_p_reference16(e);                                   // the reference's fp16 chain
             }
-            if (PROUND != 0) {                                                   // the reference's fp16 chain
-                pk = requant_p_reference2<0>(e[0], e[1], pk);
-                pk = requant_p_reference2<2>(e[2], e[3], pk);
-            }
-            p8[w4] = (int)pk;
         }
         *(v4i*)(smem + xp_wr) = p8;
         v4f vsc[DTW][4];

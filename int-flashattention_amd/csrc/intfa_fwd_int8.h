@@ -360,28 +360,27 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             // when the next block waits for it (its buffer was last read before this block's barrier)
             if (!DIAG) issue_v_slice(v_next, nb + 1, BUF ^ 1, st, NST);
             __builtin_amdgcn_sched_barrier(0);
+            if (PROUND == 0) {
 #pragma unroll
-            for (int w4 = 0; w4 < 4; ++w4) {
-                unsigned pk = 0;
-                if (PROUND == 0) {
+                for (int w4 = 0; w4 < 4; ++w4) {
+                    unsigned pk = 0;
 #pragma unroll
                     for (int b4 = 0; b4 < 4; ++b4) {
                         const float e = fast_exp2(fmaf(t[st][4 * w4 + b4], qsc, bias));   // 127 * p
                         lsum += e;
                         pk = __builtin_amdgcn_cvt_pk_u8_f32(e, b4, pk);
                     }
-                } else {
-                    // the reference's fp16 chain: fp16(p) * 127 -> fp16, + 0.5 -> fp16, truncate
-                    float e[4];
-#pragma unroll
-                    for (int b4 = 0; b4 < 4; ++b4) {
-                        e[b4] = fast_exp2(fmaf(t[st][4 * w4 + b4], qsc, bias));          // p
-                        lsum += e[b4];
-                    }
-                    pk = requant_p_reference2<0>(e[0], e[1], pk);
-                    pk = requant_p_reference2<2>(e[2], e[3], pk);
+                    p8[st][w4] = (int)pk;
                 }
-                p8[st][w4] = (int)pk;
+            } else {
+                // the reference's fp16 chain: fp16(p) * 127 -> fp16, + 0.5 -> fp16, truncate
+                float e[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    e[r] = fast_exp2(fmaf(t[st][r], qsc, bias));                          // p
+                    lsum += e[r];
+                }
+                p8[st] = requant_p_reference16(e);
             }
             asm volatile("" : "+v"(lsum));      // keep the row-sum chain inside its stage
             // the P V chain of the first d-tile advances by one MFMA as soon as this sub-tile's P8 is packed: it runs

@@ -273,27 +273,26 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
         float lsum = 0.f;
         v4i p8o;
         const float bias = (PROUND == 0 ? kLog2_127 : 0.f) - m_new;
+        if (PROUND == 0) {
 #pragma unroll
-        for (int w4 = 0; w4 < 4; ++w4) {
-            unsigned pk = 0;
-            if (PROUND == 0) {
+            for (int w4 = 0; w4 < 4; ++w4) {
+                unsigned pk = 0;
 #pragma unroll
                 for (int b4 = 0; b4 < 4; ++b4) {
                     const float e = fast_exp2(fmaf(t[4 * w4 + b4], qsc, bias));   // 127 * p
                     lsum += e;
                     pk = __builtin_amdgcn_cvt_pk_u8_f32(e, b4, pk);
                 }
-            } else {
-                float e[4];
-#pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) {
-                    e[b4] = fast_exp2(fmaf(t[4 * w4 + b4], qsc, bias));          // p
-                    lsum += e[b4];
-                }
-                pk = requant_p_reference2<0>(e[0], e[1], pk);
-                pk = requant_p_reference2<2>(e[2], e[3], pk);
+                p8o[w4] = (int)pk;
             }
-            p8o[w4] = (int)pk;
+        } else {
+            float e[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                e[r] = fast_exp2(fmaf(t[r], qsc, bias));                          // p
+                lsum += e[r];
+            }
+            p8o = requant_p_reference16(e);                                       // the reference's fp16 chain
         }
         *(v4i*)(smem + xp_wr) = p8o;
         // the chain of the first d-tile starts on this wave's own keys while the partner's P is on its way
