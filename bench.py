@@ -71,6 +71,8 @@ WORKLOADS = {
     "full_int8_B4_H32_N4096_d256": dict(variant="full", B=4, H=32, N=4096, D=256, causal=False, splits=1),
     # the headline shape with V quantised per block of 128 keys and channel (the V scales of the reference's CUDA kernel)
     "full_int8_B4_H32_N4096_d128_vblock": dict(variant="full", B=4, H=32, N=4096, D=128, causal=False, splits=1, v_block=128),
+    # the same with 64-key scale rows, the granularity of the reference's CUDA kernel (kBlockN = 64): two scale rows per key block
+    "full_int8_B4_H32_N4096_d128_vblock64": dict(variant="full", B=4, H=32, N=4096, D=128, causal=False, splits=1, v_block=64),
     # decoding against a cache: one query per head, 16384 cached keys (HBM-bound: K and V are streamed once)
     "full_int8_decode_B8_H32_Nq1_Nk16384_d128": dict(variant="full", B=8, H=32, N=1, Nk=16384, D=128, causal=False, splits="auto"),
     "full_int8_decode_B32_H32_Nq1_Nk4096_d128": dict(variant="full", B=32, H=32, N=1, Nk=4096, D=128, causal=False, splits=1),

@@ -56,7 +56,8 @@ enum {
     INTFA_ERR_SHAPE = -7,         /* batch/heads not positive, a row stride below head_dim, a (batch, head) slice of
                                      k or v spanning 4 GiB or more, or sizes that overflow 32-bit block indices */
     INTFA_ERR_SPLITS = -8,        /* num_splits out of range */
-    INTFA_ERR_VSCALE = -9         /* v_scale_block not a multiple of the key-block length, or vs_stride_blk below head_dim */
+    INTFA_ERR_VSCALE = -9         /* v_scale_block neither a multiple of the key-block length nor 64 at head_dim <= 128, or
+                                     vs_stride_blk below head_dim */
 };
 
 /*
@@ -118,7 +119,11 @@ typedef struct intfa_fwd_params {
                                  head_dim fp32 scales per block of keys (channel stride 1, row stride vs_stride_blk, batch
                                  and head strides vs_stride_b / vs_stride_h over heads_kv heads; 4-byte aligned, fp32 as in
                                  that kernel whatever scale_dtype says).  Must be a multiple of
-                                 intfa_fwd_block_n(INTFA_VARIANT_FULL_INT8, head_dim). */
+                                 intfa_fwd_block_n(INTFA_VARIANT_FULL_INT8, head_dim), or 64 at head_dim <= 128: the
+                                 granularity of the reference's kernel itself (kBlockN = 64 at head_dim 128,
+                                 csrc/flash_fwd_launch_template.h:514-519).  The softmax then still advances per 128-key
+                                 block (running maximum and P8 as intfa_fwd_block_n() says); P V is summed in int32 per
+                                 64-key half and each half is multiplied by its own scale row. */
     int32_t reserved0;        /* set to 0 */
     int64_t vs_stride_blk;    /* elements between consecutive scale rows of v_scale (>= head_dim) */
     const int32_t* seqlens_k; /* optional device array [batch]: number of keys of each batch entry, 0 <= n <= seqlen_k (a
@@ -132,7 +137,7 @@ typedef struct intfa_fwd_params {
                                  K/V group one after the other (decoding with grouped heads described as heads = heads_kv,
                                  seqlen = group * positions, see heads_kv): row r is position r % causal_rows for the causal
                                  mask.  Only with causal, full-int8, seqlen <= 64 and head_dim <= 128 (the shapes of the
-                                 decode kernel); seqlen must be a multiple of it. */
+                                 decode kernel); seqlen must be a multiple of it.  Not with v_scale_block = 64. */
     int32_t reserved1;        /* set to 0 */
 } intfa_fwd_params;
 

@@ -66,9 +66,13 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
         if (p->v_scale_block < 0) return INTFA_ERR_VSCALE;
         if (p->v_scale_block > 0) {
             const int bn = block_n_for(INTFA_VARIANT_FULL_INT8, p->head_dim);
-            if (p->v_scale_block % bn != 0 || p->vs_stride_blk < p->head_dim) return INTFA_ERR_VSCALE;
+            // a multiple of the key block, or 64 where the key block is 128: the granularity of the reference's CUDA kernel
+            // (kBlockN = 64, csrc/flash_fwd_launch_template.h:514-519), two scale rows per key block
+            const bool half_block = bn == 128 && p->v_scale_block == 64;
+            if ((p->v_scale_block % bn != 0 && !half_block) || p->vs_stride_blk < p->head_dim) return INTFA_ERR_VSCALE;
             if (reinterpret_cast<uintptr_t>(p->v_scale) & 3u) return INTFA_ERR_ALIGN;
-            k.vs_g = p->v_scale_block / bn;
+            k.vs_g = half_block ? 1 : p->v_scale_block / bn;
+            k.vs_sub = half_block ? 2 : 1;
             k.vs_sblk = p->vs_stride_blk;
         }
     }
@@ -138,7 +142,10 @@ int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dum
     sel.split = kp.num_splits > 1;
     sel.dump_s = dump_s;
     const int d = kp.head_dim;
-    if (!dump_s && decode_shaped(variant, kp.seqlen, kp.causal, d)) {
+    if (vblk && kp.vs_sub == 2) {              // (also for few query rows: the decode kernel has one scale row per block)
+        if (d == 64) return launch_full_int8_vblk64_d64(kp, sel, stream);
+        if (d == 128) return launch_full_int8_vblk64_d128(kp, sel, stream);
+    } else if (!dump_s && decode_shaped(variant, kp.seqlen, kp.causal, d)) {
         if (d == 64) return launch_decode_full_int8_d64(kp, sel, stream);
         if (d == 128) return launch_decode_full_int8_d128(kp, sel, stream);
     } else if (vblk) {
@@ -168,7 +175,7 @@ int run_forward(int variant, const intfa_fwd_params* p, int qk_bytes, int v_byte
     if (variant == INTFA_VARIANT_FULL_INT8 && p->p_round != INTFA_PROUND_RNE && p->p_round != INTFA_PROUND_REFERENCE) return INTFA_ERR_DTYPE;
     if (p->causal_rows != 0) {
         if (p->causal_rows < 0 || !p->causal || !decode_shaped(variant, kp.seqlen, kp.causal, kp.head_dim) ||
-            kp.seqlen % p->causal_rows != 0) return INTFA_ERR_SEQLEN;
+            kp.seqlen % p->causal_rows != 0 || kp.vs_sub == 2) return INTFA_ERR_SEQLEN;
         kp.causal_rows = p->causal_rows;
     }
     rc = setup_split(p, block_n_for(variant, kp.head_dim), &kp);
@@ -202,7 +209,7 @@ const char* intfa_error_string(int code) {
         case INTFA_ERR_WORKSPACE: return "workspace missing, misaligned or too small for num_splits";
         case INTFA_ERR_SHAPE: return "batch and heads must be positive and the grid must fit 31 bits";
         case INTFA_ERR_SPLITS: return "num_splits must be at most 64";
-        case INTFA_ERR_VSCALE: return "v_scale_block must be a multiple of the key-block length and vs_stride_blk at least head_dim";
+        case INTFA_ERR_VSCALE: return "v_scale_block must be a multiple of the key-block length (or 64 at head_dim <= 128) and vs_stride_blk at least head_dim";
         default: return code > 0 ? "hip error" : "unknown error";
     }
 }

@@ -72,6 +72,7 @@ struct KParams {
     int32_t kv_group;                      // query heads per K/V head (1 = every query head has its own K/V)
     int32_t pair_mblocks;                  // causal single-pass launches: one workgroup takes query blocks i and n-1-i
     int32_t vs_g;                          // blocked V scales: key blocks of the kernel per scale row (0 = scalar V scale)
+    int32_t vs_sub;                        // blocked V scales: 2 when a scale row covers 64 keys, half of the 128-key block
     int32_t causal_rows;                   // decode kernel: query positions per folded query head (0 = the row is the position)
     float qk_scale_log2;                   // sm_scale * log2(e)
 };

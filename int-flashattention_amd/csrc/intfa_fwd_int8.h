@@ -24,10 +24,14 @@ template <int D> struct FullInt8Geom {
     static constexpr int BN = 32 * NST;
 };
 
-// VBLK: V carries one scale per key block and channel (layout of the reference's CUDA kernel,
+// VBLK != 0: V carries one scale per key block and channel (layout of the reference's CUDA kernel,
 // csrc/flash_fwd_kernel_full_qi8.h:156-160) instead of one per (batch, head): the int32 P V of a block is multiplied
-// by the block's channel scales before it joins the accumulator (csrc/mask.h:313-340).
-template <int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUMP_S, bool SPLIT, bool VBLK = false>
+// by the block's channel scales before it joins the accumulator (csrc/mask.h:313-340).  VBLK == 1: a scale row covers
+// one or more whole key blocks of this kernel.  VBLK == 2: a scale row covers 64 keys, the key block of the reference's
+// CUDA kernel (kBlockN = 64 at head_dim 128, csrc/flash_fwd_launch_template.h:514-519): the softmax still advances per
+// 128-key block (the running maximum and P8 are those of intfa_fwd_block_n()), but P V is summed in int32 per 64-key
+// half and each half is multiplied by its own scale row.
+template <int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUMP_S, bool SPLIT, int VBLK = 0>
 __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T (32 bytes of head_dim each)
@@ -45,8 +49,10 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     constexpr int OFF_KS = 0;                    // two fp32 k_scale vectors
     constexpr int OFF_K = 2 * BN * 4;            // two K tiles
     constexpr int OFF_V = OFF_K + 2 * KT;        // two V tiles
-    constexpr int OFF_VS = OFF_V + 2 * VT;       // VBLK: two vectors of DV fp32 channel scales
-    constexpr int LDS_BYTES = OFF_VS + (VBLK ? 2 * DV * 4 : 0);
+    constexpr int VSUB = VBLK == 2 ? 2 : 1;      // V scale rows per key block
+    static_assert(VBLK != 2 || NST == 4, "64-key V scale rows belong to the 128-key block");
+    constexpr int OFF_VS = OFF_V + 2 * VT;       // VBLK: two vectors of VSUB * DV fp32 channel scales
+    constexpr int LDS_BYTES = OFF_VS + (VBLK ? 2 * VSUB * DV * 4 : 0);
     __shared__ __attribute__((aligned(1024))) char smem[LDS_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -198,13 +204,17 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     const bool vs_thread = VBLK && vs_c >= 0 && vs_c < DV;
     // (these scales are fp32 whatever the type of the per-token scales, as in the reference's kernel)
     const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + (vs_thread ? vs_c : 0));
-    auto load_vs = [&](int nb) __attribute__((always_inline)) -> float {
+    // (VBLK == 2: scale rows 2 nb and 2 nb + 1; the second one does not exist when the sequence ends inside the block's
+    // first half - its keys are masked, any row serves)
+    const int vs_last_row = VBLK == 2 ? (p.seqlen_k + 63) / 64 - 1 : 0;
+    auto load_vs = [&](int nb, int sub) __attribute__((always_inline)) -> float {
         if (!VBLK) return 0.f;
-        const int row = p.vs_g == 1 ? nb : nb / p.vs_g;
+        int row = p.vs_g == 1 ? nb : nb / p.vs_g;
+        if (VBLK == 2) { row = 2 * nb + sub; row = row < vs_last_row ? row : vs_last_row; }
         return Vsg[(int64_t)row * p.vs_sblk];
     };
-    const uint32_t vs_wr = OFF_VS + 4 * (vs_thread ? vs_c : 0);
-    const uint32_t vs_rd = OFF_VS + 16 * lh;       // + 4 * (32*dt + 8*a4) per read
+    const uint32_t vs_wr = OFF_VS + 4 * (vs_thread ? vs_c : 0);     // + 4 * DV for the second scale row of a block
+    const uint32_t vs_rd = OFF_VS + 16 * lh;       // + 4 * (DV * sub + 32*dt + 8*a4) per read
 
     // ---- per-lane LDS read offsets (everything else is an immediate)
     // K (A operand of S^T): lane reads row (32*st + lq), chunk (2*ks + lh), XOR-swizzled by the row
@@ -251,7 +261,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         auto load_vfrags = [&](v4i (&vf)[NST], int dt) __attribute__((always_inline)) {
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
-                if (DIAG && st > gw) continue;
+                if (DIAG && st > gw && VBLK != 2) continue;     // (VBLK == 2 multiplies every sub-tile: P8 of a hidden one is 0)
                 const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
                     (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[dt] + VB + (32 * st) * DV));
                 const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
@@ -385,15 +395,60 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             asm volatile("" : "+v"(lsum));      // keep the row-sum chain inside its stage
             // the P V chain of the first d-tile advances by one MFMA as soon as this sub-tile's P8 is packed: it runs
             // under the exponentials of the next sub-tile instead of in a burst behind the pass
-            if (!(DIAG && st > gw)) {
+            if (VBLK == 2) {                     // two chains: keys 0..63 of the block into oacc[0], keys 64..127 into oacc[1]
+                if ((st & 1) == 0) oacc[st >> 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][st], p8[st], (v16i){0}, 0, 0, 0);
+                else oacc[st >> 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][st], p8[st], oacc[st >> 1], 0, 0, 0);
+            } else if (!(DIAG && st > gw)) {
                 if (st == 0) oacc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][0], p8[0], (v16i){0}, 0, 0, 0);
                 else oacc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][st], p8[st], oacc[0], 0, 0, 0);
             }
         }
         // -------- P V on int8 MFMA: O^T[d, q] += V^T[d, key] P^T[key, q]; the chain of d-tile dt+1 is issued
         // before the accumulator update of d-tile dt, its V fragments were requested two stages earlier.
-        constexpr int VSB = BUF * DV * 4;
+        constexpr int VSB = BUF * VSUB * DV * 4;
         v4f vsc[2][4];                          // VBLK: channel scales of the d-tile being folded in / the next one
+        if constexpr (VBLK == 2) {
+            // Stage s = 2 dt + half: the int32 sum of d-tile dt over the keys 64 half .. 64 half + 63 of the block, times that
+            // half's channel scales.  Stages 0 and 1 were multiplied during pass 2; the MFMAs of stage s + 1 are issued
+            // between the quarters of the update of stage s, from stage 1 on (its accumulator is free by then).
+            constexpr int NS = 2 * DT;
+            auto load_vsc2 = [&](v4f (&dst)[4], int s2) __attribute__((always_inline)) {
+#pragma unroll
+                for (int a4 = 0; a4 < 4; ++a4)
+                    dst[a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (DV * (s2 & 1) + 32 * (s2 >> 1) + 8 * a4));
+            };
+            load_vsc2(vsc[0], 0);
+            load_vsc2(vsc[1], 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s2 = 0; s2 < NS; ++s2) {
+                const int dt = s2 >> 1, half = s2 & 1;
+                const int dtn = (s2 + 1) >> 1, halfn = (s2 + 1) & 1;      // the stage whose MFMAs are issued here
+                __builtin_amdgcn_sched_barrier(0);
+                // V fragments of d-tile dt + 2 replace those of d-tile dt once its second half has been issued
+                if (half == 1 && dt + 2 < DT) load_vfrags(vf[dt & 1], dt + 2);
+                v16i& nacc = oacc[(s2 + 1) & 1];
+#pragma unroll
+                for (int a4 = 0; a4 < 4; ++a4) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (s2 >= 1 && s2 + 1 < NS && (a4 & 1) == 0) {
+                        const int st = 2 * halfn + (a4 >> 1);
+                        if (a4 == 0) nacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[dtn & 1][st], p8[st], (v16i){0}, 0, 0, 0);
+                        else nacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[dtn & 1][st], p8[st], nacc, 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int b4 = 0; b4 < 4; ++b4) {
+                        const int r = 4 * a4 + b4;
+                        const float pv = (float)oacc[s2 & 1][r] * vsc[s2 & 1][a4][b4];
+                        if (half == 0) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(o_acc[dt][r]) : "v"(alpha), "v"(pv));
+                        else o_acc[dt][r] += pv;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (s2 + 2 < NS) load_vsc2(vsc[s2 & 1], s2 + 2);
+            }
+        } else {
         auto load_vsc = [&](v4f (&dst)[4], int dt) __attribute__((always_inline)) {
 #pragma unroll
             for (int a4 = 0; a4 < 4; ++a4) dst[a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (32 * dt + 8 * a4));
@@ -433,6 +488,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                 }
             }
         }
+        }   // VBLK != 2
         l_run = fmaf(l_run, alpha, lsum);
     };
 
@@ -444,16 +500,22 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         __syncthreads();
         const bool more = nb + 1 < nb_end;
         uint32_t ks_next = 0;
-        float vs_next = 0.f;
+        float vs_next[VSUB] = {};
         constexpr bool DIAG = decltype(diag_tag)::value;
         if (more) {
             if (DUMP_S || DIAG) issue_loads(nb + 1, BUF ^ 1);      // (a diagonal block is the last one: more == false)
             ks_next = load_ks(nb + 1);
-            if (vs_thread) vs_next = load_vs(nb + 1);
+            if (vs_thread) {
+#pragma unroll
+                for (int sub = 0; sub < VSUB; ++sub) vs_next[sub] = load_vs(nb + 1, sub);
+            }
         }
         compute(buf_tag, diag_tag, nb, more, gw, lim, lim_lo);
         if (more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
-        if (more && vs_thread) *(float*)(smem + vs_wr + (BUF ^ 1) * DV * 4) = vs_next;
+        if (more && vs_thread) {
+#pragma unroll
+            for (int sub = 0; sub < VSUB; ++sub) *(float*)(smem + vs_wr + ((BUF ^ 1) * VSUB + sub) * DV * 4) = vs_next[sub];
+        }
     };
 
     // ---- main loop: K/V tiles double-buffered in LDS, one barrier per key block.  The block on the causal
@@ -463,7 +525,10 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         {
             const uint32_t s0 = load_ks(nb_begin);
             if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
-            if (vs_thread) *(float*)(smem + vs_wr) = load_vs(nb_begin);
+            if (vs_thread) {
+#pragma unroll
+                for (int sub = 0; sub < VSUB; ++sub) *(float*)(smem + vs_wr + sub * DV * 4) = load_vs(nb_begin, sub);
+            }
         }
         // first key block that holds a key hidden from the first row of this query block (every block before it is
         // visible to all rows and runs without a mask)

@@ -18,7 +18,8 @@ def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, *,
     ``v_scale`` may also be 4-D, [Z, H, ceil(N / v_scale_block), d]: one scale per block of ``v_scale_block`` keys and
     channel, the V scales of the reference's CUDA kernel (csrc/flash_fwd_kernel_full_qi8.h:156-160), as produced by
     ``quant_perblock_channel``.  ``v_scale_block`` defaults to the kernel's key-block length (``block_n("full", d)``)
-    and must be a multiple of it.
+    and must be a multiple of it, or 64 at d <= 128 (the reference kernel's own block, kBlockN = 64,
+    csrc/flash_fwd_launch_template.h:514-519).
 
     k and v may have another length than q (and fewer heads: grouped-query attention).  With ``causal`` query row i then
     sees keys 0 .. i + Nk - Nq (mask aligned to the bottom right corner: new tokens against a cache).

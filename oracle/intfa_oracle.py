@@ -201,7 +201,10 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
     mask (stage 2), flash_atten_full_int8.py:18-25.  Returns fp32 (acc, l, m) with acc un-normalised.
     Only rows [row_lo, row_hi) are evaluated (the others keep m = -inf, l = 1, acc = 0).
     A 4-D ``v_scale`` [B,H,ceil(N/v_scale_block),d] selects the per-block, per-channel dequantisation of P V
-    (csrc/mask.h:313-340); ``v_scale_block`` must be a multiple of ``block_n``.
+    (csrc/mask.h:313-340); ``v_scale_block`` must be a multiple of ``block_n`` or divide it.  When it divides it (64-key
+    scale rows, the reference kernel's kBlockN, under a 128-key softmax block) the int32 P V is formed per scale row and
+    each partial sum is multiplied by its own row before it joins the accumulator, in ascending key order - what the
+    reference's kernel does block by block (csrc/mask.h:335-336) with the block maximum of the larger block.
     """
     B, H, N, D = q.shape
     Nk = k.shape[2]                # differs from N for cross attention / a chunk of new tokens against a cache
@@ -227,7 +230,8 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
     vs_blocked = variant == "full" and v_scale.dim() == 4
     if vs_blocked:
         v_scale_block = block_n if v_scale_block is None else v_scale_block
-        assert v_scale_block % block_n == 0 and v_scale.shape[2] == (Nk + v_scale_block - 1) // v_scale_block
+        assert (v_scale_block % block_n == 0 or block_n % v_scale_block == 0)
+        assert v_scale.shape[2] == (Nk + v_scale_block - 1) // v_scale_block
     elif variant == "full":
         vs = v_scale.float()[:, :, None, None]
     rows = torch.arange(N)
@@ -274,11 +278,17 @@ def _blocked_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: b
             a = acc[:, :, r0:r1] * alpha[..., None]                          # :56
             if variant == "full":
                 p8 = p_requant(p)                                            # :49-51
-                tmp = _int_matmul(p8, vj)                                    # :59 int32 accumulator
-                if vs_blocked:                                               # csrc/mask.h:335
-                    vs = v_scale.float()[:, :, start_n // v_scale_block][:, :, None, :]
-                tmp = tmp * vs / 127                                         # :61
-                a = a + tmp                                                  # :62
+                if vs_blocked and v_scale_block < block_n:                   # several scale rows inside this key block
+                    for c0 in range(0, kj.shape[2], v_scale_block):
+                        tmp = _int_matmul(p8[..., c0:c0 + v_scale_block], vj[:, :, c0:c0 + v_scale_block])
+                        vs = v_scale.float()[:, :, (start_n + c0) // v_scale_block][:, :, None, :]
+                        a = a + tmp * vs / 127                               # csrc/mask.h:335-336, one scale row at a time
+                else:
+                    tmp = _int_matmul(p8, vj)                                # :59 int32 accumulator
+                    if vs_blocked:                                           # csrc/mask.h:335
+                        vs = v_scale.float()[:, :, start_n // v_scale_block][:, :, None, :]
+                    tmp = tmp * vs / 127                                     # :61
+                    a = a + tmp                                              # :62
             else:
                 pl = p.to(pv_dtype).float()                                  # flash_atten_int8.py:58
                 a = a + torch.matmul(pl, vj.float())                         # :59 fp32 accumulate

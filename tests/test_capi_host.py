@@ -124,7 +124,8 @@ def _valid_block():
     (lambda p: setattr(p, "q_stride_n", 64), -7),          # rows overlap: stride below head_dim
     (lambda p: (setattr(p, "seqlen", 1 << 20), setattr(p, "k_stride_n", 1 << 13)), -7),   # a K slice of 8 GiB
     (lambda p: (setattr(p, "num_splits", 65), setattr(p, "workspace", 0x10000), setattr(p, "workspace_bytes", 1 << 40)), -8),
-    (lambda p: (setattr(p, "v_scale_block", 64), setattr(p, "vs_stride_blk", 128)), -9),    # not a multiple of the key block (128)
+    (lambda p: (setattr(p, "v_scale_block", 32), setattr(p, "vs_stride_blk", 128)), -9),    # neither a multiple of the key block (128) nor 64
+    (lambda p: (setattr(p, "v_scale_block", 192), setattr(p, "vs_stride_blk", 128)), -9),   # a multiple of 64 only
     (lambda p: (setattr(p, "v_scale_block", 128), setattr(p, "vs_stride_blk", 64)), -9),    # scale rows overlap
     (lambda p: setattr(p, "v_scale_block", -1), -9),
     (lambda p: setattr(p, "seqlen_k", -5), -3),

@@ -55,11 +55,19 @@ def test_quant_perblock_channel_strided_input():
     (1, 2, 320, 256, True, 2),
     (1, 3, 300, 128, False, 1),        # ragged length: the last scale row covers 44 keys
     (1, 2, 97, 64, True, 1),
+    # 64-key scale rows under the 128-key block: the granularity of the reference's CUDA kernel (kBlockN = 64 at
+    # head_dim 128, csrc/flash_fwd_launch_template.h:514-519); P V is summed per 64-key half
+    (1, 2, 512, 128, False, 0.5),
+    (2, 2, 384, 64, True, 0.5),
+    (1, 3, 300, 128, True, 0.5),       # ragged: the last block holds 44 keys, its second scale row does not exist
+    (1, 2, 200, 128, False, 0.5),      # the last block's second half holds 8 keys
+    (1, 2, 160, 64, False, 0.5),
+    (1, 2, 40, 128, True, 0.5),        # few query rows (the decode-shaped kernel has no 64-key rows: the general one runs)
 ])
 @pytest.mark.parametrize("p_round", ["rne", "reference"])
 def test_blocked_v_scale_matches_oracle(B, H, N, D, causal, mult, p_round):
     bn = M.block_n("full", D)
-    vsb = bn * mult
+    vsb = int(bn * mult)
     x = blocked_inputs(B, H, N, D, 80, vsb)
     sm = D ** -0.5
     o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), causal, sm, p_round=p_round,
@@ -124,15 +132,42 @@ def test_blocked_v_scale_with_grouped_heads_split_kv_and_bf16():
     assert max_abs(split, one) <= 4e-2 and mean_rel(split, one) <= 2e-2
 
 
+def test_64_key_v_scale_rows_with_grouped_heads_split_kv_decode_shapes_and_bf16():
+    B, H, H_kv, N, D = 2, 8, 2, 640, 128
+    x = blocked_inputs(B, H, N, D, 85, 64, dtype=torch.bfloat16, H_kv=H_kv)
+    sm = D ** -0.5
+    args = gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"])
+    rep = lambda t: t.repeat_interleave(H // H_kv, dim=1)
+    okw = dict(block_n=128, v_scale_block=64, out_dtype=torch.bfloat16)
+    one = M.attention_full_int8(*args, True, sm, out_dtype=torch.bfloat16, v_scale_block=64)
+    ref = O.attention_full_int8(x["q8"], rep(x["k8"]), rep(x["v8"]), x["qs"], rep(x["ks"]), rep(x["vs"]), True, sm,
+                                p_requant=O.p_requant_rne, **okw)
+    assert max_abs(one, ref) <= 3e-2 and mean_rel(one, ref) <= 3e-3          # bf16 output: 8-bit significand
+    split = M.attention_full_int8(*args, False, sm, out_dtype=torch.bfloat16, num_splits=3, p_round="reference", v_scale_block=64)
+    ref_split = O.attention_full_int8_splitkv(x["q8"], rep(x["k8"]), rep(x["v8"]), x["qs"], rep(x["ks"]), rep(x["vs"]), False,
+                                              sm, 3, **okw)
+    assert max_abs(split, ref_split) <= 3e-2 and mean_rel(split, ref_split) <= 3e-3
+    # decoding against the cache: three new tokens per head, grouped heads (no causal fold with 64-key rows), causal
+    q3, qs3 = x["q8"][:, :, -3:].contiguous(), x["qs"][:, :, -3:].contiguous()
+    dec = M.attention_full_int8(*gpu(q3, x["k8"], x["v8"], qs3, x["ks"], x["vs"]), True, sm, v_scale_block=64)
+    torch.cuda.synchronize()
+    ref_dec = O.attention_full_int8(q3, rep(x["k8"]), rep(x["v8"]), qs3, rep(x["ks"]), rep(x["vs"]), True, sm,
+                                    p_requant=O.p_requant_rne, block_n=128, v_scale_block=64)
+    assert_same_rounding(dec, ref_dec)
+
+
 def test_blocked_v_scale_small_head_dim_and_argument_checks():
     x = blocked_inputs(1, 2, 256, 32, 84, 128)
     o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, 0.2, v_scale_block=128)
     ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], False, 0.2, block_n=128,
                                 v_scale_block=128, p_requant=O.p_requant_rne)
     assert_same_rounding(o, ref)
-    with pytest.raises(RuntimeError):                          # 64 is not a multiple of the 128-key block
-        v8, vs = O.quant_perblock_channel(x["v"], 64)
-        M.attention_full_int8(*gpu(x["q8"], x["k8"], v8, x["qs"], x["ks"], vs), False, 0.2, v_scale_block=64)
+    with pytest.raises(RuntimeError):                          # 32 neither is a multiple of the 128-key block nor 64
+        v8, vs = O.quant_perblock_channel(x["v"], 32)
+        M.attention_full_int8(*gpu(x["q8"], x["k8"], v8, x["qs"], x["ks"], vs), False, 0.2, v_scale_block=32)
+    with pytest.raises(RuntimeError):                          # 192 is a multiple of 64 only
+        v8, vs = O.quant_perblock_channel(x["v"], 192)
+        M.attention_full_int8(*gpu(x["q8"], x["k8"], v8, x["qs"], x["ks"], vs), False, 0.2, v_scale_block=192)
     with pytest.raises(ValueError):                            # wrong number of scale rows
         M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"][:, :, :1]), False, 0.2, v_scale_block=128)
     with pytest.raises(ValueError):

@@ -382,6 +382,39 @@ def test_blocked_v_scale_equals_scalar_form_on_prescaled_v():
     assert torch.equal(got, want)
 
 
+def test_v_scale_rows_shorter_than_the_key_block():
+    """64-key scale rows under a 128-key softmax block (the reference kernel's kBlockN = 64 granularity of V scales)."""
+    g = torch.Generator().manual_seed(24)
+    q, k, _, _ = O.make_inputs(1, 2, 256, 16, seed=24)
+    q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k)
+    v8 = torch.randint(-15, 16, (1, 2, 256, 16), generator=g, dtype=torch.int8)
+    # (a) power-of-two factors per (64-key row, channel) equal the scalar form on V pre-multiplied by them, up to the
+    # order of two fp32 additions
+    e = torch.randint(0, 4, (1, 2, 4, 16), generator=g)
+    fac = torch.pow(2.0, e.float())
+    v8_scaled = (v8.view(1, 2, 4, 64, 16).float() * fac[:, :, :, None, :]).view(1, 2, 256, 16).to(torch.int8)
+    one = torch.ones((1, 2))
+    for causal in (False, True):
+        want = O.attention_full_int8(q8, k8, v8_scaled, qs, ks, one, causal, 0.3, block_n=128, out_dtype=torch.float32)
+        got = O.attention_full_int8(q8, k8, v8, qs, ks, fac, causal, 0.3, block_n=128, v_scale_block=64, out_dtype=torch.float32)
+        assert torch.allclose(got, want, rtol=2e-6, atol=1e-6)
+        assert not torch.allclose(got, O.attention_full_int8(q8, k8, v8, qs, ks, fac.flip(2), causal, 0.3, block_n=128,
+                                                             v_scale_block=64, out_dtype=torch.float32), rtol=1e-3)
+    # (b) one key block: the result is attention with the weights P8 / 127 over V dequantised row by row, divided by the
+    # sum of the unquantised p - evaluated densely in float64 from the definition
+    q8b, k8b, v8b, qsb, ksb = q8[:, :, :128], k8[:, :, :128], v8[:, :, :128], qs[:, :, :128], ks[:, :, :128]
+    rows = torch.rand((1, 2, 2, 16), generator=g) + 0.5
+    got = O.attention_full_int8(q8b, k8b, v8b, qsb, ksb, rows, False, 0.3, block_n=128, v_scale_block=64, out_dtype=torch.float32)
+    x = O.qk_int32(q8b, k8b).float() * qsb.float()[..., None] * ksb.float()[:, :, None, :]
+    c = float(torch.tensor(0.3, dtype=torch.float32) * torch.tensor(O.LOG2E, dtype=torch.float32))
+    m = x.max(dim=-1).values * c
+    p = torch.exp2(x * c - m[..., None])
+    p8 = O.p_requant_reference(p).double()
+    vf = v8b.double() * rows.double().repeat_interleave(64, dim=2)             # key r uses scale row r // 64
+    want = (p8 / 127) @ vf / p.double().sum(dim=-1, keepdim=True)
+    assert (got.double() - want).abs().max().item() < 1e-5 * want.abs().max().item()
+
+
 def test_blocked_v_scale_is_more_accurate_with_an_outlier_channel_burst():
     q, k, v, _ = O.make_inputs(1, 2, 256, 32, seed=15)
     v = v.clone(); v[:, :, 64:128, 5] *= 30                                     # a burst in one channel of one key block
