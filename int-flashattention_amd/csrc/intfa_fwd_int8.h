@@ -278,10 +278,11 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         v4i fr[2][KS];
         v4i vf[2][NST];
         v16i sacc[2];
-        v4f kk[2][4];
-        auto load_kk = [&](v4f (&dst)[4], int st) __attribute__((always_inline)) {
-#pragma unroll
-            for (int a4 = 0; a4 < 4; ++a4) dst[a4] = *(const v4f*)(smem + ks_rd + SB + 4 * (32 * st + 8 * a4));
+        // k_scale of the lane's keys, one quarter (4 keys) per register quad; a quad is refilled for the next sub-tile right
+        // after the quarter that consumed it (three quarters of vector work ahead of its next use)
+        v4f kk[4];
+        auto load_kk = [&](int a4, int st) __attribute__((always_inline)) {
+            kk[a4] = *(const v4f*)(smem + ks_rd + SB + 4 * (32 * st + 8 * a4));
         };
         auto qk_chain = [&](v16i& acc, const v4i (&f)[KS]) __attribute__((always_inline)) {
             acc = (v16i){0};
@@ -289,8 +290,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             for (int ks = 0; ks < KS; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[ks], qreg[ks], acc, 0, 0, 0);
         };
         load_kfrags(fr[0], 0);
-        load_kk(kk[0], 0);
-        if (1 < nact) { load_kfrags(fr[1], 1); load_kk(kk[1], 1); }
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) load_kk(a4, 0);
+        if (1 < nact) load_kfrags(fr[1], 1);
         __builtin_amdgcn_sched_barrier(0);
         qk_chain(sacc[0], fr[0]);
         // The MFMAs of sub-tile st+1 are issued one at a time between quarters of the vector work of sub-tile st: each
@@ -331,7 +333,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                 __builtin_amdgcn_sched_barrier(0);
                 float xq[4];
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) xq[b4] = (float)acc[4 * a4 + b4] * kk[st & 1][a4][b4];
+                for (int b4 = 0; b4 < 4; ++b4) xq[b4] = (float)acc[4 * a4 + b4] * kk[a4][b4];
+                if (next) load_kk(a4, st + 1);
                 if (DIAG && 32 * st + 31 > lim_lo) {           // wave-uniform: some lane of the wave has a hidden key in this sub-tile
 #pragma unroll
                     for (int b4 = 0; b4 < 4; ++b4)
@@ -344,8 +347,6 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                     mx = fmaxf(mx, x);
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
-            if (st + 2 < NST && st + 2 < nact) load_kk(kk[st & 1], st + 2);
         }
         if (DUMP_S) return;
         // V fragments of the first two d-tiles travel while the exponentials are evaluated
@@ -395,9 +396,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             asm volatile("" : "+v"(lsum));      // keep the row-sum chain inside its stage
             // the P V chain of the first d-tile advances by one MFMA as soon as this sub-tile's P8 is packed: it runs
             // under the exponentials of the next sub-tile instead of in a burst behind the pass
-            if (VBLK == 2) {                     // two chains: keys 0..63 of the block into oacc[0], keys 64..127 into oacc[1]
-                if ((st & 1) == 0) oacc[st >> 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][st], p8[st], (v16i){0}, 0, 0, 0);
-                else oacc[st >> 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][st], p8[st], oacc[st >> 1], 0, 0, 0);
+            if (VBLK == 2) {                     // keys 0..63 of the block only: the second half is a chain (and a scale row) of its own
+                if (st == 0) oacc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][0], p8[0], (v16i){0}, 0, 0, 0);
+                if (st == 1) oacc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][1], p8[1], oacc[0], 0, 0, 0);
             } else if (!(DIAG && st > gw)) {
                 if (st == 0) oacc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][0], p8[0], (v16i){0}, 0, 0, 0);
                 else oacc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[0][st], p8[st], oacc[0], 0, 0, 0);
@@ -409,16 +410,15 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         v4f vsc[2][4];                          // VBLK: channel scales of the d-tile being folded in / the next one
         if constexpr (VBLK == 2) {
             // Stage s = 2 dt + half: the int32 sum of d-tile dt over the keys 64 half .. 64 half + 63 of the block, times that
-            // half's channel scales.  Stages 0 and 1 were multiplied during pass 2; the MFMAs of stage s + 1 are issued
-            // between the quarters of the update of stage s, from stage 1 on (its accumulator is free by then).
+            // half's channel scales.  Stage 0 was multiplied during pass 2; the MFMAs of stage s + 1 are issued between the
+            // quarters of the update of stage s.
             constexpr int NS = 2 * DT;
-            auto load_vsc2 = [&](v4f (&dst)[4], int s2) __attribute__((always_inline)) {
-#pragma unroll
-                for (int a4 = 0; a4 < 4; ++a4)
-                    dst[a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (DV * (s2 & 1) + 32 * (s2 >> 1) + 8 * a4));
+            // (one quad of channel scales per quarter, refilled for the next stage right after the quarter that used it)
+            auto load_vsc2 = [&](int a4, int s2) __attribute__((always_inline)) {
+                vsc[0][a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (DV * (s2 & 1) + 32 * (s2 >> 1) + 8 * a4));
             };
-            load_vsc2(vsc[0], 0);
-            load_vsc2(vsc[1], 1);
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4) load_vsc2(a4, 0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int s2 = 0; s2 < NS; ++s2) {
@@ -431,7 +431,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
 #pragma unroll
                 for (int a4 = 0; a4 < 4; ++a4) {
                     __builtin_amdgcn_sched_barrier(0);
-                    if (s2 >= 1 && s2 + 1 < NS && (a4 & 1) == 0) {
+                    if (s2 + 1 < NS && (a4 & 1) == 0) {
                         const int st = 2 * halfn + (a4 >> 1);
                         if (a4 == 0) nacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[dtn & 1][st], p8[st], (v16i){0}, 0, 0, 0);
                         else nacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[dtn & 1][st], p8[st], nacc, 0, 0, 0);
@@ -440,13 +440,12 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
 #pragma unroll
                     for (int b4 = 0; b4 < 4; ++b4) {
                         const int r = 4 * a4 + b4;
-                        const float pv = (float)oacc[s2 & 1][r] * vsc[s2 & 1][a4][b4];
+                        const float pv = (float)oacc[s2 & 1][r] * vsc[0][a4][b4];
                         if (half == 0) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(o_acc[dt][r]) : "v"(alpha), "v"(pv));
                         else o_acc[dt][r] += pv;
                     }
+                    if (s2 + 1 < NS) load_vsc2(a4, s2 + 1);
                 }
-                __builtin_amdgcn_sched_barrier(0);
-                if (s2 + 2 < NS) load_vsc2(vsc[s2 & 1], s2 + 2);
             }
         } else {
         auto load_vsc = [&](v4f (&dst)[4], int dt) __attribute__((always_inline)) {
