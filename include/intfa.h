@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define INTFA_VERSION 6
+#define INTFA_VERSION 7
 
 /* forward variants (one entry point each, below) */
 enum { INTFA_VARIANT_FULL_INT8 = 0, INTFA_VARIANT_HALF_INT8 = 1, INTFA_VARIANT_FP16 = 2 };
@@ -56,8 +56,10 @@ enum {
     INTFA_ERR_SHAPE = -7,         /* batch/heads not positive, a row stride below head_dim, a (batch, head) slice of
                                      k or v spanning 4 GiB or more, or sizes that overflow 32-bit block indices */
     INTFA_ERR_SPLITS = -8,        /* num_splits out of range */
-    INTFA_ERR_VSCALE = -9         /* v_scale_block neither a multiple of the key-block length nor 64 at head_dim <= 128, or
+    INTFA_ERR_VSCALE = -9,        /* v_scale_block neither a multiple of the key-block length nor 64 at head_dim <= 128, or
                                      vs_stride_blk below head_dim */
+    INTFA_ERR_SCRATCH = -10       /* intfa_fwd_full_int8_static: the call's split-KV partials exceed
+                                     INTFA_STATIC_SCRATCH_BYTES, or the device index is beyond the table of 64 devices */
 };
 
 /*
@@ -168,6 +170,20 @@ size_t intfa_fwd_workspace_bytes(const intfa_fwd_params* p);
  * replaces _attention_full_int8.forward + _attn_fwd_full_int8 (flash_atten_full_int8.py:73-221);
  * native counterpart run_mha_fwd_full_qi8_ (csrc/flash_fwd_launch_template.h:503-523). */
 int intfa_fwd_full_int8(const intfa_fwd_params* p, void* stream);
+
+/* intfa_fwd_full_int8 for callers that cannot allocate device memory - code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc - and so cannot provide the workspace of a split-KV call.  It has no
+ * counterpart in the reference.  Same parameter block and results as intfa_fwd_full_int8 (bit for bit), but
+ * p->workspace and p->workspace_bytes are ignored: the split-KV partials go to a scratch array that is part of the
+ * library's device code (INTFA_STATIC_SCRATCH_BYTES bytes on each GPU the library runs on, held until the process
+ * ends).  The call works on the CURRENT device (stream must belong to it) and allocates, frees and synchronises
+ * nothing; the first call on a device looks the array's address up (make that call outside a graph capture).
+ * A call whose partials need more than INTFA_STATIC_SCRATCH_BYTES (intfa_fwd_workspace_bytes says how much) is
+ * rejected with INTFA_ERR_SCRATCH.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
+ * (different streams, or threads) race on it; calls on one stream are ordered and safe.  With num_splits <= 1 it is
+ * intfa_fwd_full_int8. */
+#define INTFA_STATIC_SCRATCH_BYTES (32u << 20)
+int intfa_fwd_full_int8_static(const intfa_fwd_params* p, void* stream);
 
 /* attention_int8(q, k, v, q_scale, k_scale, causal, sm_scale) -> o
  * replaces _attention_int8.forward + _attn_fwd_int8 (flash_atten_int8.py:68-215);

@@ -11,9 +11,10 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libintfa.so")
 
-ABI_VERSION = 6          # INTFA_VERSION of include/intfa.h this mirror was written against
+ABI_VERSION = 7          # INTFA_VERSION of include/intfa.h this mirror was written against
 INTFA_F16, INTFA_BF16, INTFA_F32 = 0, 1, 2
 PROUND_RNE, PROUND_REFERENCE = 0, 1
+STATIC_SCRATCH_BYTES = 32 << 20      # INTFA_STATIC_SCRATCH_BYTES
 
 
 class FwdParams(ctypes.Structure):
@@ -55,7 +56,7 @@ class AppendParams(ctypes.Structure):
 VARIANT_FULL_INT8, VARIANT_HALF_INT8, VARIANT_FP16 = 0, 1, 2
 
 EXPORTS = ("intfa_version", "intfa_error_string", "intfa_fwd_block_n", "intfa_fwd_workspace_bytes", "intfa_fwd_suggest_splits",
-           "intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16", "intfa_debug_qk_int32",
+           "intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16", "intfa_fwd_full_int8_static", "intfa_debug_qk_int32",
            "intfa_quant_pertoken", "intfa_quant_pertensor_workspace_bytes", "intfa_quant_pertensor",
            "intfa_quant_perblock_channel", "intfa_kvcache_append_int8")
 
@@ -83,7 +84,7 @@ def load():
     lib.intfa_fwd_suggest_splits.argtypes = [pp, ctypes.c_int, ctypes.c_int]
     lib.intfa_fwd_workspace_bytes.restype = ctypes.c_size_t
     lib.intfa_fwd_workspace_bytes.argtypes = [pp]
-    for name in ("intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16"):
+    for name in ("intfa_fwd_full_int8", "intfa_fwd_half_int8", "intfa_fwd_fp16", "intfa_fwd_full_int8_static"):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [pp, ctypes.c_void_p]

@@ -4,9 +4,36 @@
 #include "intfa_launch.h"
 #include "intfa_splitkv.h"
 
+#include <atomic>
+
 using namespace intfa;
 
+// Scratch of intfa_fwd_full_int8_static (the split-KV partials of a call that may not allocate): part of the device
+// code, so every GPU the library runs on holds its own copy at its own address until the process ends.  In host code
+// the array's name is only a handle for hipGetSymbolAddress, never an address to hand to a kernel.
+static __device__ __align__(256) unsigned char scratch[INTFA_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];          // device address of `scratch` per GPU, nullptr until looked up
+
+// Address of the scratch array on the current device; looked up once per device (any thread may be the one).
+int static_scratch_ptr(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return INTFA_ERR_SCRATCH;
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (ptr == nullptr) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);     // every thread finds the same address
+    }
+    *out = ptr;
+    return INTFA_OK;
+}
 
 constexpr int kMaxSplits = 64;
 
@@ -210,6 +237,7 @@ const char* intfa_error_string(int code) {
         case INTFA_ERR_SHAPE: return "batch and heads must be positive and the grid must fit 31 bits";
         case INTFA_ERR_SPLITS: return "num_splits must be at most 64";
         case INTFA_ERR_VSCALE: return "v_scale_block must be a multiple of the key-block length (or 64 at head_dim <= 128) and vs_stride_blk at least head_dim";
+        case INTFA_ERR_SCRATCH: return "the split-KV partials of this call exceed INTFA_STATIC_SCRATCH_BYTES (or the device index exceeds 63)";
         default: return code > 0 ? "hip error" : "unknown error";
     }
 }
@@ -239,6 +267,26 @@ int intfa_fwd_suggest_splits(const intfa_fwd_params* p, int variant, int num_cus
 
 int intfa_fwd_full_int8(const intfa_fwd_params* p, void* stream) {
     return run_forward(INTFA_VARIANT_FULL_INT8, p, 1, 1, true, true, (hipStream_t)stream);
+}
+
+int intfa_fwd_full_int8_static(const intfa_fwd_params* p, void* stream) {
+    if (p == nullptr) return INTFA_ERR_NULL;
+    intfa_fwd_params q = *p;
+    q.workspace = nullptr;
+    q.workspace_bytes = 0;
+    if (p->num_splits > 1) {
+        if (p->num_splits > kMaxSplits) return INTFA_ERR_SPLITS;
+        if (p->batch <= 0 || p->heads <= 0 || p->seqlen <= 0 || p->head_dim <= 0) return INTFA_ERR_SHAPE;
+        if (workspace_bytes_for(p) > INTFA_STATIC_SCRATCH_BYTES) return INTFA_ERR_SCRATCH;
+        void* ptr = nullptr;
+        const int rc = static_scratch_ptr(&ptr);
+        if (rc != INTFA_OK) return rc;
+        // every (split, row) of the partials is written by the forward pass before the combine pass reads it, so
+        // nothing of the previous call's contents has to be cleared
+        q.workspace = ptr;
+        q.workspace_bytes = INTFA_STATIC_SCRATCH_BYTES;
+    }
+    return run_forward(INTFA_VARIANT_FULL_INT8, &q, 1, 1, true, true, (hipStream_t)stream);
 }
 
 int intfa_fwd_half_int8(const intfa_fwd_params* p, void* stream) {
