@@ -103,8 +103,12 @@ typedef struct intfa_fwd_params {
     int32_t p_round;          /* INTFA_PROUND_* (full-int8 only) */
 
     int32_t num_splits;       /* <= 1: single pass; > 1: split-KV partials + combine (needs workspace).  The key blocks
-                                 are dealt evenly to the splits; with causal, per query block of 128 rows, the blocks
-                                 visible to it */
+                                 are dealt evenly to the splits (ceil(blocks / num_splits) consecutive blocks each).  With
+                                 causal the general kernels deal, per query block of 128 rows, the blocks VISIBLE to that
+                                 query block (ceil(visible / num_splits) each, so no split of a query block is empty);
+                                 decode-shaped full-int8 calls (seqlen <= 64, head_dim <= 128) keep the partition of the
+                                 whole key sequence also with causal.  The requantisation frame of P depends on the
+                                 ranges, so a bit-faithful CPU evaluation must use the same ones. */
     void*   workspace;        /* device scratch of at least intfa_fwd_workspace_bytes() bytes, or NULL */
     size_t  workspace_bytes;
 

@@ -221,6 +221,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
         for (int j = 0; j < DTW; ++j)
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
+                if (j == 0 && !own_tile0) continue;        // head_dim 64: waves 2 and 3 own no output tile (and no V columns)
                 const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
                     (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[j] + VB + (32 * st) * D));
                 const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
@@ -279,7 +280,8 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
 #pragma unroll
             for (int j = 0; j < DTW; ++j)
 #pragma unroll
-                for (int a4 = 0; a4 < 4; ++a4) vsc[j][a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (32 * (wave + 4 * j) + 8 * a4));
+                for (int a4 = 0; a4 < 4; ++a4)
+                    if (j > 0 || own_tile0) vsc[j][a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (32 * (wave + 4 * j) + 8 * a4));
         }
         __syncthreads();                                   // the four P8 fragments are in LDS
         v4i pall[NST];

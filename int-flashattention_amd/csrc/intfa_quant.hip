@@ -278,6 +278,7 @@ int check(const void* x, const void* q8, const void* scale, int64_t sb, int64_t 
     if ((reinterpret_cast<uintptr_t>(x) & 15u) || (reinterpret_cast<uintptr_t>(q8) & 7u) || (reinterpret_cast<uintptr_t>(scale) & 1u))
         return INTFA_ERR_ALIGN;
     if ((sb * 2) % 16 || (sh * 2) % 16 || (sn * 2) % 16) return INTFA_ERR_ALIGN;
+    if (sn < head_dim) return INTFA_ERR_SHAPE;                       // rows must not overlap (as the forward entry points require)
     qp->x = (const char*)x; qp->q8 = (char*)q8; qp->scale = (char*)scale; qp->amax = nullptr;
     qp->sb = sb * 2; qp->sh = sh * 2; qp->sn = sn * 2;
     qp->heads = heads; qp->seqlen = seqlen; qp->head_dim = head_dim;

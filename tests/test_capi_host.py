@@ -207,6 +207,7 @@ def test_quantisers_refuse_cpu_tensors_and_bad_arguments():
     assert call(x=None) == -1 and call(q8=None) == -1 and call(scale=None) == -1
     assert call(d=48) == -2 and call(dt=_capi.INTFA_F32) == -5 and call(B=0) == -7
     assert call(sn=33) == -4 and call(x=ctypes.c_void_p(8)) == -4
+    assert call(sn=24) == -7 and call(sn=16, d=32) == -7        # rows shorter than head_dim would overlap
     assert lib.intfa_quant_pertensor_workspace_bytes(4, 32) == 4 * 32 * 4
     rc = lib.intfa_quant_pertensor(one, 96 * 32, 32 * 32, 32, one, one, 2, 3, 32, 32, _capi.INTFA_F16, None, 0, None)
     assert rc == -6
