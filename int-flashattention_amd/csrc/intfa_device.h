@@ -83,6 +83,109 @@ __device__ __forceinline__ float load_scale(const char* base, int64_t idx, int d
     return ((const float*)base)[idx];
 }
 
+// ---- What every forward kernel does before its main loop: which (batch, head, query block, split) the workgroup
+// works on, which key blocks it visits, its Q fragments and scales.  One copy, shared by the four kernels.
+
+// blockIdx.x -> (batch * heads + head, index among the head's `per_head` workgroups).  Workgroups are dealt round-robin to
+// the 8 XCDs, each with its own L2: every XCD gets whole K/V heads, so the K/V tiles of a head are re-read from one L2.
+// With grouped K/V heads (kv_group query heads share one K/V head) the unit dealt to an XCD is the K/V head: all query
+// heads of a group run on the XCD whose L2 holds their K/V.
+struct WorkgroupJob { int head, rem; };
+__device__ __forceinline__ WorkgroupJob deal_workgroup(const KParams& p, int bid, int per_head) {
+    const int kv_group = p.kv_group;
+    const int per_kv = per_head * kv_group;              // workgroups per K/V head
+    const int n_kv = p.batch * p.heads / kv_group;
+    int kv_lin, r;
+    if ((n_kv & 7) == 0) {
+        const int xcd = bid & 7, slot = bid >> 3;
+        kv_lin = (slot / per_kv) * 8 + xcd;
+        r = slot % per_kv;
+    } else {
+        kv_lin = bid / per_kv;
+        r = bid % per_kv;
+    }
+    const int heads_kv = p.heads / kv_group;
+    const int bb = kv_lin / heads_kv, hk = kv_lin % heads_kv;
+    return {bb * p.heads + hk * kv_group + r / per_head, r % per_head};
+}
+
+// Number of keys of batch entry b: one length for all, or per batch (a cache filled to different lengths), clamped to
+// [0, seqlen_k] so that rows past the allocation are never addressed.
+__device__ __forceinline__ int keys_of_batch(const KParams& p, int b) {
+    int seqlen_k = p.seqlen_k;
+    if (p.seqlens_k != nullptr) {
+        const int n = p.seqlens_k[b];
+        seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
+    }
+    return seqlen_k;
+}
+
+// Key blocks [begin, end) of BN keys that a workgroup visits.  `visible_end` is the end of the range before a split
+// narrows it (the blocks that hold a key visible to some row of the workgroup).
+//   causal: the mask is aligned to the bottom right corner (csrc/mask.h:53,172 of the reference's CUDA tree): the row at
+//           position i sees keys 0 .. i + causal_off, causal_off = seqlen_k - (number of positions); pos_end is one past the
+//           workgroup's largest position.
+//   split_on: with deal_visible the VISIBLE blocks are dealt evenly to the splits (no split of a query block is empty or
+//           short); otherwise the blocks of the whole sequence are, blocks_per_split each (csrc/flash_fwd_kernel.h:503-511).
+struct KeyBlocks { int total, begin, end, visible_end; };
+template <int BN>
+__device__ __forceinline__ KeyBlocks key_block_range(int seqlen_k, bool causal, int pos_end, int causal_off, bool split_on, int n_split,
+                                                     int split, bool deal_visible, int blocks_per_split) {
+    KeyBlocks r;
+    r.total = (seqlen_k + BN - 1) / BN;
+    r.begin = 0;
+    r.end = r.total;
+    if (causal) {
+        const int e = (pos_end + causal_off + BN - 1) / BN;
+        r.end = e < 0 ? 0 : (e < r.total ? e : r.total);
+    }
+    r.visible_end = r.end;
+    if (split_on) {
+        const int per = deal_visible ? (r.end + n_split - 1) / n_split : blocks_per_split;
+        r.begin = split * per;
+        const int e = r.begin + per;
+        r.end = e < r.end ? e : r.end;
+    }
+    return r;
+}
+
+// int8 Q fragments of query row q_ld (B operand of S^T = K Q^T): 16 bytes per k-step of 32, the half lh of the lane.
+template <int KS>
+__device__ __forceinline__ void load_q8_fragments(v4i (&qreg)[KS], const KParams& p, int b, int h, int q_ld, int lh) {
+    const char* qrow = p.q + b * p.q_sb + h * p.q_sh + (int64_t)q_ld * p.q_sn;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qreg[ks] = *(const v4i*)(qrow + ks * 32 + lh * 16);
+}
+// q_scale of query row q_ld times sm_scale * log2(e): the factor between S * k_scale and the exponent of exp2.
+__device__ __forceinline__ float load_q_scale_log2(const KParams& p, int b, int h, int q_ld) {
+    return load_scale(p.q_scale, b * p.qs_sb + h * p.qs_sh + (int64_t)q_ld * p.qs_sn, p.scale_dtype) * p.qk_scale_log2;
+}
+
+// k_scale of the keys of one (batch, K/V head): fetched as raw bits (one key per thread, ahead of the block that uses
+// them) and converted to fp32 when stored to LDS.  Keys past the end read the last key's scale; they are masked later.
+struct KScaleSource {
+    const char* base;
+    int stride, dtype, seqlen_k;
+    __device__ __forceinline__ KScaleSource(const KParams& p, int b, int hk, int seqlen_k_) {
+        const int esize = p.scale_dtype == 2 ? 4 : 2;
+        base = p.k_scale + (b * p.ks_sb + hk * p.ks_sh) * esize;
+        stride = (int)(p.ks_sn * esize);
+        dtype = p.scale_dtype;
+        seqlen_k = seqlen_k_;
+    }
+    __device__ __forceinline__ uint32_t load(int key) const {
+        key = key < seqlen_k ? key : seqlen_k - 1;
+        const char* src = base + (int64_t)key * stride;
+        if (dtype == 2) return *(const uint32_t*)src;
+        return (uint32_t)*(const uint16_t*)src;
+    }
+    __device__ __forceinline__ float cvt(uint32_t raw) const {
+        if (dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+        if (dtype == 1) return __builtin_bit_cast(float, raw << 16);
+        return __builtin_bit_cast(float, raw);
+    }
+};
+
 // ---- LDS swizzles.  A tile row is ROW_BYTES bytes; its 16-byte chunks are XOR-permuted with a function of the
 // row so that the rows touched together by one LDS access cycle (64 banks x 4 bytes = 256 bytes: 16 lanes of a
 // 16-byte read, 32 lanes of an 8-byte read) fall into different bank groups.  Every function depends on the low

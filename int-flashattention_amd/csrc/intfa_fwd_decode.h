@@ -50,69 +50,34 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const int n_mblk = (p.seqlen + kDecodeRows - 1) / kDecodeRows;
     const int n_split = SPLIT ? p.num_splits : 1;
     const int per_head = n_mblk * n_split;
-    const int n_heads = p.batch * p.heads;
-    const int bid = blockIdx.x;
+    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x, per_head);
+    const int rem = wg.rem, head = wg.head;
     const int kv_group = p.kv_group;
-    const int per_kv = per_head * kv_group;
-    const int n_kv = n_heads / kv_group;
-    int head, rem;
-    {
-        int kv_lin, r;
-        if ((n_kv & 7) == 0) {
-            const int xcd = bid & 7, slot = bid >> 3;
-            kv_lin = (slot / per_kv) * 8 + xcd;
-            r = slot % per_kv;
-        } else {
-            kv_lin = bid / per_kv;
-            r = bid % per_kv;
-        }
-        const int heads_kv = p.heads / kv_group;
-        const int bb = kv_lin / heads_kv, hk_ = kv_lin % heads_kv;
-        head = bb * p.heads + hk_ * kv_group + r / per_head;
-        rem = r % per_head;
-    }
     const int mb = rem / n_split, split = rem % n_split;
     const int b = head / p.heads, h = head % p.heads;
     const int hk = h / kv_group;
 
-    // number of keys of this batch entry: one length for all, or per batch (a cache filled to different lengths)
-    int seqlen_k = p.seqlen_k;
-    if (p.seqlens_k != nullptr) {            // clamped to [0, seqlen_k]: rows past the allocation are never addressed
-        const int n = p.seqlens_k[b];
-        seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
-    }
-    const int nb_total = (seqlen_k + BN - 1) / BN;
+    const int seqlen_k = keys_of_batch(p, b);
     // causal: row i sees keys 0 .. i + causal_off (mask aligned to the bottom right corner as in the general kernels: a few
     // new tokens against a cache); blocks past the last row's limit are not visited
     // (causal_rows: the rows hold several query heads of one K/V group, causal_rows positions each; a row's position is
     // then row % causal_rows and a 32-row block can hold every position)
     const int fold = p.causal_rows;
     const int causal_off = seqlen_k - (fold ? fold : p.seqlen);
-    int nb_begin = 0, nb_end = nb_total;
-    if (p.causal) {
-        const int last_pos = fold ? fold : mb * kDecodeRows + kDecodeRows;       // one past the largest position in this block
-        const int e = (last_pos + causal_off + BN - 1) / BN;
-        nb_end = e < 0 ? 0 : (e < nb_total ? e : nb_total);
-    }
-    const int causal_end = nb_end;                        // (before the split range narrows it)
-    if (SPLIT) {                                           // csrc/flash_fwd_kernel.h:503-511
-        nb_begin = split * p.blocks_per_split;
-        const int e = nb_begin + p.blocks_per_split;
-        nb_end = e < nb_end ? e : nb_end;
-    }
+    // (a split takes blocks_per_split blocks of the whole key range, masked or not: every row of a decode-shaped problem
+    // sees nearly all keys)
+    const KeyBlocks kb = key_block_range<BN>(seqlen_k, p.causal != 0, fold ? fold : mb * kDecodeRows + kDecodeRows, causal_off, SPLIT,
+                                             n_split, split, false, p.blocks_per_split);
+    const int nb_total = kb.total, nb_begin = kb.begin, nb_end = kb.end;
+    const int causal_end = kb.visible_end;                // (before the split range narrows it)
     const int q_row = mb * kDecodeRows + lq;
     const bool q_valid = q_row < p.seqlen;
     const int q_ld = q_valid ? q_row : p.seqlen - 1;
 
     // ---- Q fragment (B operand of S^T = K Q^T), the same 32 rows in every wave
     v4i qreg[KS];
-    {
-        const char* qrow = p.q + b * p.q_sb + h * p.q_sh + (int64_t)q_ld * p.q_sn;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qreg[ks] = *(const v4i*)(qrow + ks * 32 + lh * 16);
-    }
-    const float qs = load_scale(p.q_scale, b * p.qs_sb + h * p.qs_sh + (int64_t)q_ld * p.qs_sn, p.scale_dtype);
-    const float qsc = qs * p.qk_scale_log2;
+    load_q8_fragments<KS>(qreg, p, b, h, q_ld, lh);
+    const float qsc = load_q_scale_log2(p, b, h, q_ld);
 
     float m_run = -INFINITY, l_run = 0.f;        // l_run: this wave's keys only
     float o_acc[DTW][16];
@@ -135,21 +100,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
         issue_tile_load<D, SWZ_V8, BN>(v_rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane);
     };
     // k_scale of a block: thread t < 128 fetches the scale of key t; converted to fp32 when stored to LDS
-    const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
-    const char* Ksg = p.k_scale + (b * p.ks_sb + hk * p.ks_sh) * ks_esize;
-    const int ks_stride = (int)(p.ks_sn * ks_esize);
-    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
-        int key = nb * BN + (tid & (BN - 1));
-        key = key < seqlen_k ? key : seqlen_k - 1;                  // keys past the end are masked later
-        const char* src = Ksg + (int64_t)key * ks_stride;
-        if (p.scale_dtype == 2) return *(const uint32_t*)src;
-        return (uint32_t)*(const uint16_t*)src;
-    };
-    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float {
-        if (p.scale_dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
-        if (p.scale_dtype == 1) return __builtin_bit_cast(float, raw << 16);
-        return __builtin_bit_cast(float, raw);
-    };
+    const KScaleSource ks_src(p, b, hk, seqlen_k);
+    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t { return ks_src.load(nb * BN + (tid & (BN - 1))); };
+    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
     // VBLK: fp32 channel scales of a key block; thread 128 + c fetches channel c
     const int vs_c = tid - 128;
     const bool vs_thread = VBLK && vs_c >= 0 && vs_c < D;

@@ -66,29 +66,9 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
     // workgroup then walks the same number of key blocks and the launch has no tail of light workgroups.
     const bool pair = CAUSAL && !SPLIT && p.pair_mblocks != 0;
     const int per_head = (pair ? n_mblk / 2 : n_mblk * n_split) * NHALF;
-    const int n_heads = p.batch * p.heads;
-    const int bid = blockIdx.x;
-    // With grouped K/V heads (kv_group query heads share one K/V head) the unit dealt to an XCD is the K/V head: all
-    // query heads of a group run on the XCD whose L2 holds their K/V.
+    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x, per_head);
+    const int rem = wg.rem, head = wg.head;
     const int kv_group = p.kv_group;
-    const int per_kv = per_head * kv_group;              // workgroups per K/V head
-    const int n_kv = n_heads / kv_group;
-    int head, rem;
-    {
-        int kv_lin, r;
-        if ((n_kv & 7) == 0) {
-            const int xcd = bid & 7, slot = bid >> 3;
-            kv_lin = (slot / per_kv) * 8 + xcd;
-            r = slot % per_kv;
-        } else {
-            kv_lin = bid / per_kv;
-            r = bid % per_kv;
-        }
-        const int heads_kv = p.heads / kv_group;
-        const int bb = kv_lin / heads_kv, hk = kv_lin % heads_kv;
-        head = bb * p.heads + hk * kv_group + r / per_head;
-        rem = r % per_head;
-    }
     const int half = rem % NHALF;                // column half of this workgroup (0 when the columns are not split)
     const int mb_idx = (rem / NHALF) / n_split;
     const int split = (rem / NHALF) % n_split;
@@ -102,28 +82,12 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
     const int hk = h / kv_group;                     // K/V head of this query head
     // ragged sequence lengths are handled as in the full-int8 kernel (zero-filled copies, masked last block, rows past
     // the end computed on clamped inputs and not stored)
-    // number of keys of this batch entry: one length for all, or per batch (a cache filled to different lengths)
-    int seqlen_k = p.seqlen_k;
-    if (p.seqlens_k != nullptr) {            // clamped to [0, seqlen_k]: rows past the allocation are never addressed
-        const int n = p.seqlens_k[b];
-        seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
-    }
-    const int nb_total = (seqlen_k + BN - 1) / BN;
+    const int seqlen_k = keys_of_batch(p, b);
     // causal mask aligned to the bottom right corner as in the full-int8 kernel: row i sees keys 0 .. i + causal_off
     const int causal_off = seqlen_k - p.seqlen;
-    int nb_begin = 0, nb_end = nb_total;
-    if (CAUSAL) {
-        const int e = (mb * kBlockM + kBlockM + causal_off + BN - 1) / BN;
-        nb_end = e < 0 ? 0 : (e < nb_total ? e : nb_total);
-    }
-    if (SPLIT) {
-        // non-causal: the key blocks of the sequence are dealt evenly to the splits (csrc/flash_fwd_kernel.h:503-511);
-        // causal: the blocks VISIBLE to this query block are, so that no split of a query block is empty or short
-        const int per = CAUSAL ? (nb_end + n_split - 1) / n_split : p.blocks_per_split;
-        nb_begin = split * per;
-        const int e = nb_begin + per;
-        nb_end = e < nb_end ? e : nb_end;
-    }
+    const KeyBlocks kb = key_block_range<BN>(seqlen_k, CAUSAL, mb * kBlockM + kBlockM, causal_off, SPLIT, n_split, split, CAUSAL,
+                                             p.blocks_per_split);
+    const int nb_total = kb.total, nb_begin = kb.begin, nb_end = kb.end;
     const int q_row = mb * kBlockM + wave * 32 + lq;
     const bool q_valid = q_row < p.seqlen;
     const int q_ld = q_valid ? q_row : p.seqlen - 1;     // row read for lanes past the end
@@ -158,22 +122,11 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
         issue_tile_load<KROW, SWZ_K, BN>(k_rsrc, (uint32_t)(nb * BN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane);
         issue_tile_load<VROW, SWZ_V16, BN>(v_rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane);
     };
-    const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
-    const char* Ksg = QK_INT8 ? p.k_scale + (b * p.ks_sb + hk * p.ks_sh) * ks_esize : nullptr;
-    const int ks_stride = (int)(p.ks_sn * ks_esize);
+    const KScaleSource ks_src(p, b, hk, seqlen_k);
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
-        if (!QK_INT8 || tid >= BN) return 0u;
-        int key = nb * BN + tid;
-        key = key < seqlen_k ? key : seqlen_k - 1;                                    // keys past the end are masked later
-        const char* src = Ksg + (int64_t)key * ks_stride;
-        if (p.scale_dtype == 2) return *(const uint32_t*)src;
-        return (uint32_t)*(const uint16_t*)src;
+        return (!QK_INT8 || tid >= BN) ? 0u : ks_src.load(nb * BN + tid);
     };
-    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float {
-        if (p.scale_dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
-        if (p.scale_dtype == 1) return __builtin_bit_cast(float, raw << 16);
-        return __builtin_bit_cast(float, raw);
-    };
+    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
 
     // ---- per-lane LDS read offsets
     const int k_swz = swz_k<KROW>(lq) & (KCH - 1);

@@ -67,29 +67,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     // workgroup then walks the same number of key blocks and the launch has no tail of light workgroups.
     const bool pair = CAUSAL && !SPLIT && p.pair_mblocks != 0;
     const int per_head = pair ? n_mblk / 2 : n_mblk * n_split;
-    const int n_heads = p.batch * p.heads;
-    const int bid = blockIdx.x;
-    // With grouped K/V heads (kv_group query heads share one K/V head) the unit dealt to an XCD is the K/V head: all
-    // query heads of a group run on the XCD whose L2 holds their K/V.
+    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x, per_head);
+    const int head = wg.head, rem = wg.rem;
     const int kv_group = p.kv_group;
-    const int per_kv = per_head * kv_group;              // workgroups per K/V head
-    const int n_kv = n_heads / kv_group;
-    int head, rem;
-    {
-        int kv_lin, r;
-        if ((n_kv & 7) == 0) {
-            const int xcd = bid & 7, slot = bid >> 3;
-            kv_lin = (slot / per_kv) * 8 + xcd;
-            r = slot % per_kv;
-        } else {
-            kv_lin = bid / per_kv;
-            r = bid % per_kv;
-        }
-        const int heads_kv = p.heads / kv_group;
-        const int bb = kv_lin / heads_kv, hk = kv_lin % heads_kv;
-        head = bb * p.heads + hk * kv_group + r / per_head;
-        rem = r % per_head;
-    }
     const int mb_idx = rem / n_split;
     const int split = rem % n_split;
     const int njobs = pair ? 2 : 1;
@@ -105,42 +85,21 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     // Sequence lengths that are not a multiple of the block sizes: the copies of K/V rows past the end return zeros
     // (bounds-checked buffer loads), the last key block runs the masked code instance, query rows past the end are
     // computed on clamped inputs and not stored.
-    // number of keys of this batch entry: one length for all, or per batch (a cache filled to different lengths)
-    int seqlen_k = p.seqlen_k;
-    if (p.seqlens_k != nullptr) {            // clamped to [0, seqlen_k]: rows past the allocation are never addressed
-        const int n = p.seqlens_k[b];
-        seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
-    }
-    const int nb_total = (seqlen_k + BN - 1) / BN;
-    // Causal mask aligned to the bottom right corner (csrc/mask.h:53,172 of the reference's CUDA tree): query row i sees
-    // keys 0 .. i + causal_off.  Equal lengths (the reference's Python API) give causal_off = 0.
+    const int seqlen_k = keys_of_batch(p, b);
+    // Causal mask aligned to the bottom right corner: query row i sees keys 0 .. i + causal_off.  Equal lengths (the
+    // reference's Python API) give causal_off = 0.
     const int causal_off = seqlen_k - p.seqlen;
-    int nb_begin = 0, nb_end = nb_total;
-    if (CAUSAL) {                                          // blocks that hold a key visible to the last row of this query block
-        const int e = (mb * kBlockM + kBlockM + causal_off + BN - 1) / BN;
-        nb_end = e < 0 ? 0 : (e < nb_total ? e : nb_total);
-    }
-    if (SPLIT) {
-        // non-causal: the key blocks of the sequence are dealt evenly to the splits (csrc/flash_fwd_kernel.h:503-511);
-        // causal: the blocks VISIBLE to this query block are, so that no split of a query block is empty or short
-        const int per = CAUSAL ? (nb_end + n_split - 1) / n_split : p.blocks_per_split;
-        nb_begin = split * per;
-        const int e = nb_begin + per;
-        nb_end = e < nb_end ? e : nb_end;
-    }
+    const KeyBlocks kb = key_block_range<BN>(seqlen_k, CAUSAL, mb * kBlockM + kBlockM, causal_off, SPLIT, n_split, split, CAUSAL,
+                                             p.blocks_per_split);
+    const int nb_total = kb.total, nb_begin = kb.begin, nb_end = kb.end;
     const int q_row = mb * kBlockM + wave * 32 + lq;     // this lane's query row
     const bool q_valid = q_row < p.seqlen;
     const int q_ld = q_valid ? q_row : p.seqlen - 1;     // row read for lanes past the end
 
     // ---- Q fragment (B operand of S^T = K Q^T): 16 bytes per k-step, resident for the whole kernel.
     v4i qreg[KS];
-    {
-        const char* qrow = p.q + b * p.q_sb + h * p.q_sh + (int64_t)q_ld * p.q_sn;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qreg[ks] = *(const v4i*)(qrow + ks * 32 + lh * 16);
-    }
-    const float qs = DUMP_S ? 1.f : load_scale(p.q_scale, b * p.qs_sb + h * p.qs_sh + (int64_t)q_ld * p.qs_sn, p.scale_dtype);
-    const float qsc = qs * p.qk_scale_log2;
+    load_q8_fragments<KS>(qreg, p, b, h, q_ld, lh);
+    const float qsc = DUMP_S ? p.qk_scale_log2 : load_q_scale_log2(p, b, h, q_ld);
 
     float m_run = -INFINITY, l_run = 0.f;
     float o_acc[DT][16];
@@ -181,23 +140,12 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
                 issue_tile_part<DV, SWZ_V8, BN>(rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane, it);
     };
     // k_scale of a block: thread t < 128 fetches the scale of key t; converted to fp32 when stored to LDS
-    const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
-    const char* Ksg = p.k_scale + (b * p.ks_sb + hk * p.ks_sh) * ks_esize;
+    const KScaleSource ks_src(p, b, hk, seqlen_k);
     const int ks_key = tid & (BN - 1);
-    const int ks_stride = (int)(p.ks_sn * ks_esize);
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {           // raw bits
-        if (DUMP_S) return 0u;
-        int key = nb * BN + ks_key;
-        key = key < seqlen_k ? key : seqlen_k - 1;                                    // keys past the end are masked later
-        const char* src = Ksg + (int64_t)key * ks_stride;
-        if (p.scale_dtype == 2) return *(const uint32_t*)src;
-        return (uint32_t)*(const uint16_t*)src;
+        return DUMP_S ? 0u : ks_src.load(nb * BN + ks_key);
     };
-    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float {
-        if (p.scale_dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
-        if (p.scale_dtype == 1) return __builtin_bit_cast(float, raw << 16);
-        return __builtin_bit_cast(float, raw);
-    };
+    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
     // VBLK: channel scales of a key block; thread 128 + c fetches the scale of this workgroup's channel c.  A scale
     // row covers vs_g key blocks.
     const int vs_c = tid - 128;

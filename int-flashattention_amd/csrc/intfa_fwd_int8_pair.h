@@ -49,27 +49,9 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
     const int n_split = SPLIT ? p.num_splits : 1;
     const bool pair = CAUSAL && !SPLIT && p.pair_mblocks != 0;
     const int per_head = pair ? n_mblk / 2 : n_mblk * n_split;
-    const int n_heads = p.batch * p.heads;
-    const int bid = blockIdx.x;
+    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x, per_head);
+    const int rem = wg.rem, head = wg.head;
     const int kv_group = p.kv_group;
-    const int per_kv = per_head * kv_group;
-    const int n_kv = n_heads / kv_group;
-    int head, rem;
-    {
-        int kv_lin, r;
-        if ((n_kv & 7) == 0) {
-            const int xcd = bid & 7, slot = bid >> 3;
-            kv_lin = (slot / per_kv) * 8 + xcd;
-            r = slot % per_kv;
-        } else {
-            kv_lin = bid / per_kv;
-            r = bid % per_kv;
-        }
-        const int heads_kv = p.heads / kv_group;
-        const int bb = kv_lin / heads_kv, hk = kv_lin % heads_kv;
-        head = bb * p.heads + hk * kv_group + r / per_head;
-        rem = r % per_head;
-    }
     const int mb_idx = rem / n_split;
     const int split = rem % n_split;
     const int njobs = pair ? 2 : 1;
@@ -81,38 +63,20 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
     const int b = head / p.heads, h = head % p.heads;
     const int hk = h / kv_group;
 
-    int seqlen_k = p.seqlen_k;
-    if (p.seqlens_k != nullptr) {                // clamped to [0, seqlen_k]: rows past the allocation are never addressed
-        const int n = p.seqlens_k[b];
-        seqlen_k = n < 0 ? 0 : (n < seqlen_k ? n : seqlen_k);
-    }
-    const int nb_total = (seqlen_k + BN - 1) / BN;
-    // causal mask aligned to the bottom right corner (csrc/mask.h:53,172): query row i sees keys 0 .. i + causal_off
+    const int seqlen_k = keys_of_batch(p, b);
+    // causal mask aligned to the bottom right corner: query row i sees keys 0 .. i + causal_off
     const int causal_off = seqlen_k - p.seqlen;
-    int nb_begin = 0, nb_end = nb_total;
-    if (CAUSAL) {
-        const int e = (mb * kBlockM + kBlockM + causal_off + BN - 1) / BN;
-        nb_end = e < 0 ? 0 : (e < nb_total ? e : nb_total);
-    }
-    if (SPLIT) {                                 // same ranges as fwd_full_int8_kernel
-        const int per = CAUSAL ? (nb_end + n_split - 1) / n_split : p.blocks_per_split;
-        nb_begin = split * per;
-        const int e = nb_begin + per;
-        nb_end = e < nb_end ? e : nb_end;
-    }
+    const KeyBlocks kb = key_block_range<BN>(seqlen_k, CAUSAL, mb * kBlockM + kBlockM, causal_off, SPLIT, n_split, split, CAUSAL,
+                                             p.blocks_per_split);
+    const int nb_total = kb.total, nb_begin = kb.begin, nb_end = kb.end;
     const int q_row = mb * kBlockM + rw * 32 + lq;
     const bool q_valid = q_row < p.seqlen;
     const int q_ld = q_valid ? q_row : p.seqlen - 1;
 
     // ---- Q fragment (B operand of S^T = K Q^T), resident
     v4i qreg[KS];
-    {
-        const char* qrow = p.q + b * p.q_sb + h * p.q_sh + (int64_t)q_ld * p.q_sn;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qreg[ks] = *(const v4i*)(qrow + ks * 32 + lh * 16);
-    }
-    const float qs = load_scale(p.q_scale, b * p.qs_sb + h * p.qs_sh + (int64_t)q_ld * p.qs_sn, p.scale_dtype);
-    const float qsc = qs * p.qk_scale_log2;
+    load_q8_fragments<KS>(qreg, p, b, h, q_ld, lh);
+    const float qsc = load_q_scale_log2(p, b, h, q_ld);
 
     float m_run = -INFINITY, l_run = 0.f;        // l_run: this wave's keys only
     float o_acc[DT][16];
@@ -137,22 +101,10 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
         issue_tile_load<D, SWZ_K, BN>(t_rsrc, (uint32_t)(nb * BN) * t_sn, t_sn, t_lds + buf * KT, rw, t_lane);
     };
     // k_scale of a block: thread t < 64 fetches the scale of key t; converted to fp32 when stored to LDS
-    const int ks_esize = p.scale_dtype == 2 ? 4 : 2;
-    const char* Ksg = p.k_scale + (b * p.ks_sb + hk * p.ks_sh) * ks_esize;
+    const KScaleSource ks_src(p, b, hk, seqlen_k);
     const int ks_key = tid & (BN - 1);
-    const int ks_stride = (int)(p.ks_sn * ks_esize);
-    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {           // raw bits
-        int key = nb * BN + ks_key;
-        key = key < seqlen_k ? key : seqlen_k - 1;                                    // keys past the end are masked later
-        const char* src = Ksg + (int64_t)key * ks_stride;
-        if (p.scale_dtype == 2) return *(const uint32_t*)src;
-        return (uint32_t)*(const uint16_t*)src;
-    };
-    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float {
-        if (p.scale_dtype == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
-        if (p.scale_dtype == 1) return __builtin_bit_cast(float, raw << 16);
-        return __builtin_bit_cast(float, raw);
-    };
+    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t { return ks_src.load(nb * BN + ks_key); };   // raw bits
+    auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
     // VBLK: thread 256 + c fetches the fp32 scale of channel c of the key block's scale row (vs_g key blocks per row)
     const int vs_c = tid - 256;
     const bool vs_thread = VBLK && vs_c >= 0;
