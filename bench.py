@@ -59,6 +59,9 @@ WORKLOADS = {
     "half_int8_B8_H32_N2048_d128_causal": dict(variant="half", B=8, H=32, N=2048, D=128, causal=True, splits=1),
     "half_int8_B4_H32_N4096_d128": dict(variant="half", B=4, H=32, N=4096, D=128, causal=False, splits=1),
     "fp16_B4_H32_N4096_d128": dict(variant="fp", B=4, H=32, N=4096, D=128, causal=False, splits=1),
+    # head_dim 256 of the two 16-bit-PV variants (eight-wave workgroups, two waves per 32 query rows)
+    "half_int8_B4_H32_N4096_d256": dict(variant="half", B=4, H=32, N=4096, D=256, causal=False, splits=1),
+    "fp16_B4_H32_N4096_d256": dict(variant="fp", B=4, H=32, N=4096, D=256, causal=False, splits=1),
     "full_int8_B1_H32_N16384_d128_causal_splitkv": dict(variant="full", B=1, H=32, N=16384, D=128, causal=True, splits=2,
                                                         k_outlier_frac=0.01),
     "full_int8_B1_H32_N16384_d128_causal": dict(variant="full", B=1, H=32, N=16384, D=128, causal=True, splits=1,

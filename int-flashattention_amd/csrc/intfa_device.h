@@ -264,7 +264,7 @@ __device__ __forceinline__ void issue_tile_part(v4i rsrc, uint32_t tile_off, uin
     const uint32_t m0v = lds_tile + (uint32_t)i * 1024u;
     const uint32_t soff = tile_off + (uint32_t)(i * T::RPI) * row_stride;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(m0v), "v"(ln.off[it % T::NV]), "s"(rsrc), "s"(soff) : "memory", "m0");
+                 :: "s"(m0v), "v"(ln.off[it % T::NV]), "s"(rsrc), "s"(soff) : "memory");
 }
 template <int ROW_BYTES, int SWZ, int ROWS>
 __device__ __forceinline__ void issue_tile_load(v4i rsrc, uint32_t tile_off, uint32_t row_stride, uint32_t lds_tile,

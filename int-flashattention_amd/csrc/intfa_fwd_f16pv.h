@@ -30,8 +30,9 @@ __device__ __forceinline__ v8bf pack_p_bf16(const float* e) {
 // QK_INT8: int8 Q/K with scales (half-int8) or 16-bit Q/K (fp16/bf16 variant).  IO_DT: type of V, P and the output
 // (and of Q/K when !QK_INT8): 0 fp16, 1 bf16.
 // Output columns one workgroup produces.  At head_dim 256 a full-width workgroup needs 128 fp32 output registers per lane:
-// one wave per SIMD and spills.  The columns are split over two workgroups that each redo Q K^T and the softmax and
-// multiply P with their half of V.
+// one wave per SIMD and spills.  This kernel can split the columns over two workgroups that each redo Q K^T and the
+// softmax and multiply P with their half of V; the library does not instantiate it at head_dim 256 any more -
+// fwd_f16pv_pair_kernel (intfa_fwd_f16pv_pair.h) divides the work between two waves of one workgroup instead.
 template <int D> struct F16PvGeom {
     static constexpr int DV = D <= 128 ? D : 128;
     static constexpr int NHALF = D / DV;
