@@ -256,6 +256,10 @@ __device__ __forceinline__ v4i make_rsrc(const void* base, uint32_t bytes) {
     return r;
 }
 // Issues wave instruction number `it` (0 .. NINST/4 - 1) of this wave's share of one tile copy.
+// The statement overwrites M0 and cannot say so: the compiler keeps M0 reserved on this target, warns about a clobber
+// entry for it and ignores it.  Nothing the compiler generates in these kernels reads M0 (no LDS-DMA builtins, GWS,
+// relative moves or interpolation), and every copy sets it afresh.  tile_off and row_stride must be wave-uniform values
+// the compiler can see as such (kernel arguments, readfirstlane results): they end up in scalar operands.
 template <int ROW_BYTES, int SWZ, int ROWS>
 __device__ __forceinline__ void issue_tile_part(v4i rsrc, uint32_t tile_off, uint32_t row_stride, uint32_t lds_tile,
                                                 int wave, const TileLoadLane<ROW_BYTES, SWZ, ROWS>& ln, int it) {
