@@ -37,7 +37,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_f16pv_pair_kernel(const K
     // LDS map (bytes)
     constexpr int OFF_KS = 0;                    // two fp32 k_scale vectors
     constexpr int OFF_XM = OFF_KS + 2 * BN * 4;  // row maxima (and, in the epilogue, row sums): [wave][32]
-    constexpr int OFF_XP = OFF_XM + 8 * 32 * 4;  // 16-bit P fragments: [wave][lane] x 32 bytes
+    constexpr int OFF_XP = OFF_XM + 8 * 32 * 4;  // 16-bit P fragments: [16-key step][wave][lane] x 16 bytes
     constexpr int OFF_K = (OFF_XP + 8 * 64 * 32 + 1023) & ~1023;
     constexpr int OFF_V = OFF_K + 2 * KT;
     constexpr int LDS_BYTES = OFF_V + 2 * VT;
@@ -137,7 +137,9 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_f16pv_pair_kernel(const K
     const uint32_t ks_rd = OFF_KS + 4 * 32 * hf + 16 * lh;                 // + 32 * a4 per read
     const uint32_t ks_wr = OFF_KS + 4 * (tid & (BN - 1));
     const uint32_t xm_wr = OFF_XM + 4 * (wave * 32 + lq), xm_rd = OFF_XM + 4 * ((wave ^ 4) * 32 + lq);
-    const uint32_t xp_wr = OFF_XP + 32 * (wave * 64 + lane), xp_rd = OFF_XP + 32 * ((wave ^ 4) * 64 + lane);
+    // (a lane's two fragments lie 8 KiB apart, so that consecutive lanes write consecutive 16 bytes: no bank conflicts)
+    constexpr uint32_t XP_U = 8 * 64 * 16;
+    const uint32_t xp_wr = OFF_XP + 16 * (wave * 64 + lane), xp_rd = OFF_XP + 16 * ((wave ^ 4) * 64 + lane);
 
     auto mfma16 = [&](v4i a, v4i b2, v16f c) __attribute__((always_inline)) -> v16f {
         if (IO_DT == 0) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b2), c, 0, 0, 0);
@@ -225,7 +227,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_f16pv_pair_kernel(const K
         for (int u = 0; u < 2; ++u)
             pfo[u] = IO_DT == 0 ? __builtin_bit_cast(v4i, pack_p_f16(e + 8 * u)) : __builtin_bit_cast(v4i, pack_p_bf16(e + 8 * u));
         *(v4i*)(smem + xp_wr) = pfo[0];
-        *(v4i*)(smem + xp_wr + 16) = pfo[1];
+        *(v4i*)(smem + xp_wr + XP_U) = pfo[1];
         l_run = fmaf(l_run, alpha, lsum);
         // the first d-tile is rescaled and its chain starts on this wave's own keys while the partner's P is on its way
 #pragma unroll
@@ -240,7 +242,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_f16pv_pair_kernel(const K
         }
         __syncthreads();                         // ---- B3
         pfp[0] = *(const v4i*)(smem + xp_rd);
-        pfp[1] = *(const v4i*)(smem + xp_rd + 16);
+        pfp[1] = *(const v4i*)(smem + xp_rd + XP_U);
         // K fragments of the next block (other buffer): the k-steps of stage dt + 1 are requested when those of stage dt
         // have been issued
         v4i fr[KPS];
