@@ -195,7 +195,7 @@ enum { SWZ_K = 0, SWZ_V8 = 1, SWZ_V16 = 2 };
 template <int ROW_BYTES> __device__ __forceinline__ int swz_k(int row) {
     if (ROW_BYTES >= 256) return row & 15;                           // every row starts at bank 0
     if (ROW_BYTES == 128) return (row & 7) ^ ((row >> 3) & 1);       // rows r, r+8 share banks: flip bit 0
-    return (row >> 1) & 3;                                           // 64-byte rows: 4 rows per 256 bytes
+    return (row >> 2) & 3;                                           // 64-byte rows: rows r, r+4, r+8, r+12 share banks
 }
 // int8 V rows read by ds_read_b64_tr_b8: a 16-lane group touches rows {0,1,2,3,8,9,10,11} + 4h of a sub-tile.
 template <int ROW_BYTES> __device__ __forceinline__ int swz_v8(int row) {
