@@ -278,6 +278,41 @@ __device__ __forceinline__ void issue_tile_load(v4i rsrc, uint32_t tile_off, uin
     for (int it = 0; it < T::NINST / 4; ++it) issue_tile_part<ROW_BYTES, SWZ, ROWS>(rsrc, tile_off, row_stride, lds_tile, wave, ln, it);
 }
 
+// ---- 16-bit output rows through LDS.  In the accumulator layout a lane holds four consecutive columns of ONE row per
+// register quad, so a direct store writes 8-byte pieces of 32 different rows per instruction and every 64-byte line
+// of the output is touched by several partial writes.  Each wave therefore stages its 32 rows x NCOL columns in a
+// private LDS region (rows of NCOL * 2 bytes, 16-byte chunks XOR-permuted by the row so that neither the 8-byte
+// writes nor the 16-byte reads meet in a bank) and writes them out with 16 bytes per lane: a row's NCOL * 2 bytes are
+// contiguous in one store instruction.  The region must be dead tile memory: a workgroup barrier lies between the last
+// tile read of any wave and the first out_stage_put.
+template <int NCOL> struct OutStage {
+    static constexpr int RS = NCOL * 2;                  // bytes per staged row
+    static constexpr int CH = RS / 16;                   // 16-byte chunks per row
+    static constexpr int RPB = RS >= 256 ? 1 : 256 / RS; // rows per 256 bytes (one pass over the banks)
+    static constexpr int BYTES = 32 * RS;                // per wave
+    static constexpr int LPR = RS / 16, RPI = 64 / LPR;  // lanes per row / rows per store instruction
+    static_assert(NCOL == 64 || NCOL == 128, "staging is laid out for 128- and 256-byte rows");
+    static __device__ __forceinline__ int key(int row) { return (row / RPB) & (CH - 1); }
+};
+// four 16-bit values (columns d0 .. d0 + 3, d0 a multiple of 4) of the wave's row `row`
+template <int NCOL>
+__device__ __forceinline__ void out_stage_put(char* stage, int row, int d0, v2i bits) {
+    using S = OutStage<NCOL>;
+    *(v2i*)(stage + row * S::RS + ((((d0 * 2) >> 4) ^ S::key(row)) << 4) + ((d0 * 2) & 15)) = bits;
+}
+// g_row0: global address of the wave's first row (column offset applied); rows_valid: how many of the 32 rows exist
+template <int NCOL>
+__device__ __forceinline__ void out_stage_flush(const char* stage, char* g_row0, int64_t row_stride, int rows_valid, int lane) {
+    using S = OutStage<NCOL>;
+    const int sub = lane / S::LPR, ch = lane % S::LPR;
+#pragma unroll
+    for (int j = 0; j < 32 / S::RPI; ++j) {
+        const int row = j * S::RPI + sub;
+        const v4i x = *(const v4i*)(stage + row * S::RS + ((ch ^ S::key(row)) << 4));
+        if (row < rows_valid) *(v4i*)(g_row0 + row * row_stride + ch * 16) = x;
+    }
+}
+
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {   // round-to-nearest-even
     uint32_t u = __builtin_bit_cast(uint32_t, f);
     u += 0x7fffu + ((u >> 16) & 1u);

@@ -354,27 +354,38 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
         }
         return;
     }
-    char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn + half * DV * 2;
-    if (q_valid) {
+    {
+    // 16-bit rows go out through LDS (whole lines per store instruction); the tiles are dead once every wave is here
+    static_assert(4 * OutStage<DV>::BYTES <= LDS_BYTES, "output staging fits the tile memory");
+    __syncthreads();
+    // (an opaque copy of the lane index: the staging addresses depend on the lane only and would otherwise be computed
+    // ahead of the main loop and held in registers through it)
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int lq_e = lane_e & 31, lh_e = lane_e >> 5;
+    char* stage = smem + wave * OutStage<DV>::BYTES;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int a4 = 0; a4 < 4; ++a4) {
-            const int d0 = 32 * dt + 8 * a4 + 4 * lh;
+            const int d0 = 32 * dt + 8 * a4 + 4 * lh_e;
             if (IO_DT == 0) {
                 v4h o;
 #pragma unroll
                 for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(any_key ? o_acc[dt][4 * a4 + b4] * inv : 0.f);
-                *(v4h*)(orow + d0 * 2) = o;
+                out_stage_put<DV>(stage, lq_e, d0, __builtin_bit_cast(v2i, o));
             } else {
                 v4s o;
 #pragma unroll
                 for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(any_key ? o_acc[dt][4 * a4 + b4] * inv : 0.f);
-                *(v4s*)(orow + d0 * 2) = o;
+                out_stage_put<DV>(stage, lq_e, d0, __builtin_bit_cast(v2i, o));
             }
         }
-    if (pe->lse != nullptr && lh == 0 && half == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
-    }   // q_valid
+    const int row0 = mb * kBlockM + wave * 32;
+    out_stage_flush<DV>(stage, pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)row0 * pe->o_sn + half * DV * 2, pe->o_sn,
+                        e_seqlen - row0, lane_e);
+    if (q_valid && pe->lse != nullptr && lh == 0 && half == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
+    }
     }   // job
 #endif  // __HIP_DEVICE_COMPILE__
 }

@@ -334,26 +334,37 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_f16pv_pair_kernel(const K
                 }
             if (lh == 0 && hf == 0) pe->lse_part[row] = lse;
         }
-    } else if (q_valid) {
-        char* orow = pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)q_row * pe->o_sn + hf * DVW * 2;
+    } else {
+        // 16-bit rows go out through LDS (whole lines per store instruction), staged in the tile memory: every wave has
+        // passed the barrier of the row-sum exchange, so no tile is read any more
+        static_assert(OFF_K + 8 * OutStage<DVW>::BYTES <= LDS_BYTES, "output staging fits the tile memory");
+        // (an opaque copy of the lane index: the staging addresses depend on the lane only and would otherwise be computed
+    // ahead of the main loop and held in registers through it)
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int lq_e = lane_e & 31, lh_e = lane_e >> 5;
+    char* stage = smem + OFF_K + wave * OutStage<DVW>::BYTES;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int a4 = 0; a4 < 4; ++a4) {
-                const int d0 = 32 * dt + 8 * a4 + 4 * lh;
+                const int d0 = 32 * dt + 8 * a4 + 4 * lh_e;
                 if (IO_DT == 0) {
                     v4h o;
 #pragma unroll
                     for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(any_key ? o_acc[dt][4 * a4 + b4] * inv : 0.f);
-                    *(v4h*)(orow + d0 * 2) = o;
+                    out_stage_put<DVW>(stage, lq_e, d0, __builtin_bit_cast(v2i, o));
                 } else {
                     v4s o;
 #pragma unroll
                     for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(any_key ? o_acc[dt][4 * a4 + b4] * inv : 0.f);
-                    *(v4s*)(orow + d0 * 2) = o;
+                    out_stage_put<DVW>(stage, lq_e, d0, __builtin_bit_cast(v2i, o));
                 }
             }
-        if (pe->lse != nullptr && lh == 0 && hf == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
+        const int row0 = mb * kBlockM + rw * 32;
+        out_stage_flush<DVW>(stage, pe->out + eb * pe->o_sb + eh * pe->o_sh + (int64_t)row0 * pe->o_sn + hf * DVW * 2, pe->o_sn,
+                             e_seqlen - row0, lane_e);
+        if (q_valid && pe->lse != nullptr && lh == 0 && hf == 0) pe->lse[((int64_t)eb * e_heads + eh) * e_seqlen + q_row] = lse;
     }
     }   // job
 #endif  // __HIP_DEVICE_COMPILE__
