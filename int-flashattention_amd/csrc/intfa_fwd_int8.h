@@ -544,6 +544,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     if constexpr (!DUMP_S) {
     // 16-bit rows go out through LDS (whole lines per store instruction); the tiles are dead once every wave is here
     static_assert(4 * OutStage<DV>::BYTES <= LDS_BYTES, "output staging fits the tile memory");
+    // (the last block's copy slices ran against an empty resource: they fetch nothing but still write zeros into the
+    // other tile buffers, asynchronously - every wave awaits its own before the barrier)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     // (an opaque copy of the lane index: the staging addresses depend on the lane only and would otherwise be computed
     // ahead of the main loop and held in registers through it)
