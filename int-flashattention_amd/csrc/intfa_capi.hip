@@ -73,9 +73,9 @@ int make_kparams(const intfa_fwd_params* p, int qk_bytes, int v_bytes, bool need
     k.k_sb = p->k_stride_b * qk_bytes; k.k_sh = p->k_stride_h * qk_bytes; k.k_sn = p->k_stride_n * qk_bytes;
     if (v_bytes > 0) {
         if (p->v == nullptr || p->out == nullptr) return INTFA_ERR_NULL;
-        if (!aligned16(p->v) || (reinterpret_cast<uintptr_t>(p->out) & 7u)) return INTFA_ERR_ALIGN;
+        if (!aligned16(p->v) || !aligned16(p->out)) return INTFA_ERR_ALIGN;     // (the output rows are stored 16 bytes per lane)
         if ((p->v_stride_n * v_bytes) % 16 || (p->v_stride_b * v_bytes) % 16 || (p->v_stride_h * v_bytes) % 16) return INTFA_ERR_ALIGN;
-        if ((p->o_stride_n * 2) % 8 || (p->o_stride_b * 2) % 8 || (p->o_stride_h * 2) % 8) return INTFA_ERR_ALIGN;
+        if ((p->o_stride_n * 2) % 16 || (p->o_stride_b * 2) % 16 || (p->o_stride_h * 2) % 16) return INTFA_ERR_ALIGN;
         if (p->v_stride_n < p->head_dim || p->o_stride_n < p->head_dim) return INTFA_ERR_SHAPE;
         k.v = (const char*)p->v; k.out = (char*)p->out;
         k.v_sb = p->v_stride_b * v_bytes; k.v_sh = p->v_stride_h * v_bytes; k.v_sn = p->v_stride_n * v_bytes;

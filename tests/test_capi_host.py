@@ -116,6 +116,8 @@ def _valid_block():
     (lambda p: setattr(p, "seqlen", 0), -3),
     (lambda p: setattr(p, "k", 0x10008), -4),
     (lambda p: setattr(p, "q_stride_n", 120), -4),
+    (lambda p: setattr(p, "out", 0x10008), -4),            # the output rows are stored 16 bytes per lane
+    (lambda p: setattr(p, "o_stride_n", 132), -4),         # 264 bytes: a multiple of 8 only
     (lambda p: setattr(p, "scale_dtype", 7), -5),
     (lambda p: setattr(p, "io_dtype", 2), -5),
     (lambda p: setattr(p, "num_splits", 4), -6),          # splits requested without a workspace
