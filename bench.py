@@ -79,6 +79,9 @@ WORKLOADS = {
     # decoding against a cache: one query per head, 16384 cached keys (HBM-bound: K and V are streamed once)
     "full_int8_decode_B8_H32_Nq1_Nk16384_d128": dict(variant="full", B=8, H=32, N=1, Nk=16384, D=128, causal=False, splits="auto"),
     "full_int8_decode_B32_H32_Nq1_Nk4096_d128": dict(variant="full", B=32, H=32, N=1, Nk=4096, D=128, causal=False, splits=1),
+    # the same decode shape for the two variants with a 16-bit V cache (int8 or 16-bit K cache)
+    "half_int8_decode_B32_H32_Nq1_Nk4096_d128": dict(variant="half", B=32, H=32, N=1, Nk=4096, D=128, causal=False, splits=1),
+    "fp16_decode_B32_H32_Nq1_Nk4096_d128": dict(variant="fp", B=32, H=32, N=1, Nk=4096, D=128, causal=False, splits=1),
     # the input quantisers (HBM-bound): Q/K per token, V per (batch, head)
     "quant_pertoken_B4_H32_N4096_d128": dict(variant="quant_token", B=4, H=32, N=4096, D=128, causal=False, splits=1),
     "quant_pertensor_B4_H32_N4096_d128": dict(variant="quant_tensor", B=4, H=32, N=4096, D=128, causal=False, splits=1),
@@ -366,18 +369,21 @@ def main():
             "median_launch_ms": other_round["median_launch_ms"],
             "slowdown_vs_timed_rounding": other_round["avg_launch_ms"] / kern_ms}
     if decode:
-        # one pass over the cached K and V (int8) and their scales; Q, O and the split partials are a rounding error
+        # one pass over the cached K and V and the k scales; Q, O and the split partials are a rounding error
         sb = 2 if dt != torch.float32 else 4
-        alg_bytes = B * H * Nk * (2 * D + sb) + B * H * N * D * 3
+        k_bytes = 1 if variant in ("full", "half") else 2
+        v_bytes = 1 if variant == "full" else 2
+        alg_bytes = B * H * Nk * (D * (k_bytes + v_bytes) + (sb if variant != "fp" else 0)) + B * H * N * D * (k_bytes + 2)
         gbs = alg_bytes / (kern_ms * 1e-3) / 1e9
-        out["metric"] = "decode attention: cached K+V bytes streamed per second (full-int8, one query per head)"
+        vname = {"full": "full-int8", "half": "half-int8", "fp": "fp16"}[variant]
+        out["metric"] = f"decode attention: cached K+V bytes streamed per second ({vname}, one query per head)"
         out["value"], out["unit"] = alg_bytes / (ms_step * 1e-3) / 1e9, "GB/s"
         out["config"]["seqlen_k"] = Nk
         out["config"]["bytes_per_step"] = alg_bytes
         out.pop("pct_int8_peak")
         out["roofline"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                            "traffic": traffic_of(args.workload)[0], "traffic_source": traffic_of(args.workload)[1],
-                           "kernel": "fwd_decode_full_int8_kernel", "avg_launch_ms": kern_ms, "median_launch_ms": kern_med_ms,
+                           "kernel": "fwd_decode_full_int8_kernel" if variant == "full" else "fwd_decode_f16pv_kernel", "avg_launch_ms": kern_ms, "median_launch_ms": kern_med_ms,
                            "launch_includes": "forward kernel" + (" + split-KV combine kernel" if splits != 1 else "")}
     if parity is not None:
         out["parity"] = parity

@@ -123,8 +123,8 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
     # Few queries per head with grouped K/V heads (decoding): the g query heads of a group become g*N rows of ONE head,
     # so that a group streams its K/V once instead of g times.  Pure re-striding: same memory, same results per row.
     g = H // H_kv
-    # (with the causal mask only where the kernel can be told the position of a row: the decode-shaped full-int8 calls)
-    fold_rows = 2 * BLOCK if not causal else (64 if variant == "full" and dk <= 128 and p.v_scale_block != 64 else 0)
+    # (with the causal mask only where the kernel can be told the position of a row: the decode-shaped calls)
+    fold_rows = 2 * BLOCK if not causal else (64 if dk <= 128 and p.v_scale_block != 64 else 0)
     if g > 1 and g * N <= fold_rows and _can_fold(q_, N) and (variant == "fp" or _can_fold(q_scale, N)):
         if causal:
             p.causal_rows = N

@@ -150,14 +150,14 @@ int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t str
     return e == hipSuccess ? INTFA_OK : (int)e;
 }
 
-// Few query rows per head (decoding against a cache): the full-int8 pass runs the kernel whose waves share the keys of a
-// block instead of each taking 32 query rows.
-// (Head_dim 256 stays with the general kernel: its key block is 64 there, the decode kernel's is 128, and the block
-// length is part of the arithmetic that intfa_fwd_block_n() promises.)
+// Few query rows per head (decoding against a cache): the pass runs a kernel whose waves share the keys of a block
+// instead of each taking 32 query rows (intfa_fwd_decode.h, intfa_fwd_decode_f16pv.h).
+// (Head_dim 256 stays with the general kernels.)
 constexpr int kDecodeMaxRows = 2 * kDecodeRows;
 bool decode_shaped(int variant, int seqlen, int causal, int head_dim) {
-    (void)causal;      // the decode kernel masks too: a few new tokens against a cache
-    return variant == INTFA_VARIANT_FULL_INT8 && seqlen <= kDecodeMaxRows && head_dim <= 128;
+    (void)variant;
+    (void)causal;      // the decode kernels mask too: a few new tokens against a cache
+    return seqlen <= kDecodeMaxRows && head_dim <= 128;
 }
 
 int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dump_s, hipStream_t stream) {
@@ -173,8 +173,16 @@ int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dum
         if (d == 64) return launch_full_int8_vblk64_d64(kp, sel, stream);
         if (d == 128) return launch_full_int8_vblk64_d128(kp, sel, stream);
     } else if (!dump_s && decode_shaped(variant, kp.seqlen, kp.causal, d)) {
-        if (d == 64) return launch_decode_full_int8_d64(kp, sel, stream);
-        if (d == 128) return launch_decode_full_int8_d128(kp, sel, stream);
+        if (variant == INTFA_VARIANT_FULL_INT8) {
+            if (d == 64) return launch_decode_full_int8_d64(kp, sel, stream);
+            if (d == 128) return launch_decode_full_int8_d128(kp, sel, stream);
+        } else if (variant == INTFA_VARIANT_HALF_INT8) {
+            if (d == 64) return launch_decode_half_int8_d64(kp, sel, stream);
+            if (d == 128) return launch_decode_half_int8_d128(kp, sel, stream);
+        } else {
+            if (d == 64) return launch_decode_fp16_d64(kp, sel, stream);
+            if (d == 128) return launch_decode_fp16_d128(kp, sel, stream);
+        }
     } else if (vblk) {
         if (d == 64) return launch_full_int8_vblk_d64(kp, sel, stream);
         if (d == 128) return launch_full_int8_vblk_d128(kp, sel, stream);
@@ -230,7 +238,7 @@ const char* intfa_error_string(int code) {
         case INTFA_OK: return "ok";
         case INTFA_ERR_NULL: return "a required pointer is NULL";
         case INTFA_ERR_HEAD_DIM: return "head_dim must be 64, 128 or 256";
-        case INTFA_ERR_SEQLEN: return "seqlen must be positive, seqlen_k not negative, causal_rows only on causal decode-shaped full-int8 calls";
+        case INTFA_ERR_SEQLEN: return "seqlen must be positive, seqlen_k not negative, causal_rows only on causal decode-shaped calls";
         case INTFA_ERR_ALIGN: return "pointers and row/head/batch strides must be 16-byte aligned";
         case INTFA_ERR_DTYPE: return "unknown dtype enum";
         case INTFA_ERR_WORKSPACE: return "workspace missing, misaligned or too small for num_splits";
@@ -251,9 +259,12 @@ int intfa_fwd_suggest_splits(const intfa_fwd_params* p, int variant, int num_cus
     if (p->seqlen <= 0 || p->seqlen_k < 0) return INTFA_ERR_SEQLEN;
     if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256) return INTFA_ERR_HEAD_DIM;
     const int cus = num_cus > 0 ? num_cus : 256;
-    const int64_t slots = 2ll * cus;                                           // two workgroups per compute unit
+    int64_t slots = 2ll * cus;                                                 // two workgroups per compute unit
     int64_t wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kBlockM - 1) / kBlockM);
-    if (decode_shaped(variant, p->seqlen, p->causal, p->head_dim)) wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kDecodeRows - 1) / kDecodeRows);
+    if (decode_shaped(variant, p->seqlen, p->causal, p->head_dim)) {
+        wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kDecodeRows - 1) / kDecodeRows);
+        if (variant != INTFA_VARIANT_FULL_INT8 && p->head_dim == 128) slots = cus;   // 16-bit V tiles of two steps: one workgroup per compute unit
+    }
     else if (p->head_dim == 256) wgs *= 2;     // full-int8: eight-wave workgroups, one per compute unit; the others: column halves
     if (wgs * 5 >= slots * 4) return 1;                                        // at least 80 % of the slots are used anyway
     const int seqlen_k = p->seqlen_k > 0 ? p->seqlen_k : p->seqlen;
