@@ -79,6 +79,7 @@ WORKLOADS = {
     # decoding against a cache: one query per head, 16384 cached keys (HBM-bound: K and V are streamed once)
     "full_int8_decode_B8_H32_Nq1_Nk16384_d128": dict(variant="full", B=8, H=32, N=1, Nk=16384, D=128, causal=False, splits="auto"),
     "full_int8_decode_B32_H32_Nq1_Nk4096_d128": dict(variant="full", B=32, H=32, N=1, Nk=4096, D=128, causal=False, splits=1),
+    "full_int8_decode_B32_H32_Nq1_Nk4096_d256": dict(variant="full", B=32, H=32, N=1, Nk=4096, D=256, causal=False, splits=1),
     # the same decode shape for the two variants with a 16-bit V cache (int8 or 16-bit K cache)
     "half_int8_decode_B32_H32_Nq1_Nk4096_d128": dict(variant="half", B=32, H=32, N=1, Nk=4096, D=128, causal=False, splits=1),
     "fp16_decode_B32_H32_Nq1_Nk4096_d128": dict(variant="fp", B=32, H=32, N=1, Nk=4096, D=128, causal=False, splits=1),

@@ -142,9 +142,9 @@ typedef struct intfa_fwd_params {
     int32_t causal_rows;      /* 0, or the number of query positions when the row axis holds several query heads of one
                                  K/V group one after the other (decoding with grouped heads described as heads = heads_kv,
                                  seqlen = group * positions, see heads_kv): row r is position r % causal_rows for the causal
-                                 mask.  Only with causal, seqlen <= 64 and head_dim <= 128 (the shapes of the decode
-                                 kernels, any of the three variants); seqlen must be a multiple of it.  Not with
-                                 v_scale_block = 64. */
+                                 mask.  Only with causal and the shapes of the decode kernels: seqlen <= 64 and
+                                 head_dim <= 128 (any variant; not with v_scale_block = 64), or head_dim 256 in the
+                                 full-int8 variant with v_scale_block = 0.  seqlen must be a multiple of it. */
     int32_t reserved1;        /* set to 0 */
 } intfa_fwd_params;
 

@@ -152,12 +152,12 @@ int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t str
 
 // Few query rows per head (decoding against a cache): the pass runs a kernel whose waves share the keys of a block
 // instead of each taking 32 query rows (intfa_fwd_decode.h, intfa_fwd_decode_f16pv.h).
-// (Head_dim 256 stays with the general kernels.)
+// Head_dim 256: the full-int8 variant with one V scale per (batch, head); its other forms and the 16-bit V caches of the
+// other variants (their tiles of a step do not fit the LDS twice) stay with the general kernels.
 constexpr int kDecodeMaxRows = 2 * kDecodeRows;
-bool decode_shaped(int variant, int seqlen, int causal, int head_dim) {
-    (void)variant;
-    (void)causal;      // the decode kernels mask too: a few new tokens against a cache
-    return seqlen <= kDecodeMaxRows && head_dim <= 128;
+bool decode_shaped(int variant, int seqlen, int head_dim, bool blocked_v_scales) {
+    if (seqlen > kDecodeMaxRows) return false;
+    return head_dim <= 128 || (head_dim == 256 && variant == INTFA_VARIANT_FULL_INT8 && !blocked_v_scales);
 }
 
 int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dump_s, hipStream_t stream) {
@@ -172,10 +172,11 @@ int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dum
     if (vblk && kp.vs_sub == 2) {              // (also for few query rows: the decode kernel has one scale row per block)
         if (d == 64) return launch_full_int8_vblk64_d64(kp, sel, stream);
         if (d == 128) return launch_full_int8_vblk64_d128(kp, sel, stream);
-    } else if (!dump_s && decode_shaped(variant, kp.seqlen, kp.causal, d)) {
+    } else if (!dump_s && decode_shaped(variant, kp.seqlen, d, vblk)) {
         if (variant == INTFA_VARIANT_FULL_INT8) {
             if (d == 64) return launch_decode_full_int8_d64(kp, sel, stream);
             if (d == 128) return launch_decode_full_int8_d128(kp, sel, stream);
+            if (d == 256) return launch_decode_full_int8_d256(kp, sel, stream);
         } else if (variant == INTFA_VARIANT_HALF_INT8) {
             if (d == 64) return launch_decode_half_int8_d64(kp, sel, stream);
             if (d == 128) return launch_decode_half_int8_d128(kp, sel, stream);
@@ -209,7 +210,7 @@ int run_forward(int variant, const intfa_fwd_params* p, int qk_bytes, int v_byte
     if (rc != INTFA_OK) return rc;
     if (variant == INTFA_VARIANT_FULL_INT8 && p->p_round != INTFA_PROUND_RNE && p->p_round != INTFA_PROUND_REFERENCE) return INTFA_ERR_DTYPE;
     if (p->causal_rows != 0) {
-        if (p->causal_rows < 0 || !p->causal || !decode_shaped(variant, kp.seqlen, kp.causal, kp.head_dim) ||
+        if (p->causal_rows < 0 || !p->causal || !decode_shaped(variant, kp.seqlen, kp.head_dim, kp.vs_g > 0) ||
             kp.seqlen % p->causal_rows != 0 || kp.vs_sub == 2) return INTFA_ERR_SEQLEN;
         kp.causal_rows = p->causal_rows;
     }
@@ -261,9 +262,10 @@ int intfa_fwd_suggest_splits(const intfa_fwd_params* p, int variant, int num_cus
     const int cus = num_cus > 0 ? num_cus : 256;
     int64_t slots = 2ll * cus;                                                 // two workgroups per compute unit
     int64_t wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kBlockM - 1) / kBlockM);
-    if (decode_shaped(variant, p->seqlen, p->causal, p->head_dim)) {
+    if (decode_shaped(variant, p->seqlen, p->head_dim, variant == INTFA_VARIANT_FULL_INT8 && p->v_scale_block > 0)) {
         wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kDecodeRows - 1) / kDecodeRows);
-        if (variant != INTFA_VARIANT_FULL_INT8 && p->head_dim == 128) slots = cus;   // 16-bit V tiles of two steps: one workgroup per compute unit
+        // 128 KiB of tiles and more: one workgroup per compute unit
+        if ((variant != INTFA_VARIANT_FULL_INT8 && p->head_dim == 128) || p->head_dim == 256) slots = cus;
     }
     else if (p->head_dim == 256) wgs *= 2;     // full-int8: eight-wave workgroups, one per compute unit; the others: column halves
     if (wgs * 5 >= slots * 4) return 1;                                        // at least 80 % of the slots are used anyway

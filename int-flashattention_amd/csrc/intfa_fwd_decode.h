@@ -13,24 +13,32 @@
 // The int32 sums run over the same 128 keys as in the general kernel, so results agree with it up to the order of the
 // fp32 additions of the row sums.  K/V tiles are double-buffered in LDS and the whole next tile is requested at the
 // start of a block (the data comes from HBM, not from a cache shared with other query blocks).
+// Head_dim 256: the general kernel's key block is 64 there (fwd_full_int8_pair_kernel), so a 128-key step of this
+// kernel covers TWO blocks A (waves 0, 1) and B (waves 2, 3): after the one exchange of partial maxima every wave knows
+// m_A = max(m, max_A), m_B = max(m_A, max_B) and both factors alpha_A = 2^(m - m_A), alpha_B = 2^(m_A - m_B); each wave
+// requantises its keys in its own block's frame, and an output tile is updated as
+// O = (O alpha_A + P8_A V_A) alpha_B + P8_B V_B with one int32 sum per block - the blocks' arithmetic of that kernel.
 #pragma once
 #include "intfa_device.h"
 #include "intfa_launch.h"
 
 namespace intfa {
 
-// Head dims 64 and 128 (the key block of the general kernel is 128 there too, so both kernels evaluate the same blocks).
+// Head dims 64 and 128 (the key block of the general kernel is 128 there too, so both kernels evaluate the same blocks)
+// and 256 (two 64-key blocks per step; one scale per (batch, head) only).
 template <int D, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool SPLIT, bool VBLK>
-__global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const KParams p) {
-    static_assert(D == 64 || D == 128, "the decode kernel shares the 128-key block of the general kernel");
+__global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_int8_kernel(const KParams p) {
+    static_assert(D == 64 || D == 128 || (D == 256 && !VBLK), "head dims 64, 128, and 256 without blocked V scales");
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T
     constexpr int DT = D / 32;                   // 32-wide output tiles along head_dim; wave w owns tiles w, w+4, ...
     constexpr int DTW = (DT + 3) / 4;            // output tiles per wave
     constexpr int NST = 4, BN = 32 * NST;        // one 32-key sub-tile per wave
+    constexpr int NBS = D == 256 ? 2 : 1;        // key blocks (of the arithmetic) per step
+    constexpr int BNB = BN / NBS;                // key block of the arithmetic: intfa_fwd_block_n()
     constexpr int KT = BN * D, VT = BN * D;      // bytes of one K / V tile
     constexpr int CH = D / 16;                   // 16-byte chunks per row
-    constexpr int SWM = (CH < 8 ? CH : 8) - 1;   // swizzle mask of V rows
+    constexpr int SWM = CH - 1;                  // swizzle mask of V rows
     // LDS map (bytes)
     constexpr int OFF_KS = 0;                            // two fp32 k_scale vectors
     constexpr int OFF_XM = 2 * BN * 4;                   // 4 waves x 32 rows fp32: partial row maxima / row sums
@@ -66,10 +74,10 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const int causal_off = seqlen_k - (fold ? fold : p.seqlen);
     // (a split takes blocks_per_split blocks of the whole key range, masked or not: every row of a decode-shaped problem
     // sees nearly all keys)
-    const KeyBlocks kb = key_block_range<BN>(seqlen_k, p.causal != 0, fold ? fold : mb * kDecodeRows + kDecodeRows, causal_off, SPLIT,
+    const KeyBlocks kb = key_block_range<BNB>(seqlen_k, p.causal != 0, fold ? fold : mb * kDecodeRows + kDecodeRows, causal_off, SPLIT,
                                              n_split, split, false, p.blocks_per_split);
-    const int nb_total = kb.total, nb_begin = kb.begin, nb_end = kb.end;
-    const int causal_end = kb.visible_end;                // (before the split range narrows it)
+    const int nb_begin = kb.begin, nb_end = kb.end;         // in blocks of BNB keys
+    const int key_end = nb_end * BNB < seqlen_k ? nb_end * BNB : seqlen_k;      // one past the last key of the range
     const int q_row = mb * kDecodeRows + lq;
     const bool q_valid = q_row < p.seqlen;
     const int q_ld = q_valid ? q_row : p.seqlen - 1;
@@ -96,12 +104,12 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const auto v_lane = tile_load_lane<D, SWZ_V8, BN>(v_sn, wave, lane);
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
     auto issue_loads = [&](int nb, int buf) __attribute__((always_inline)) {
-        issue_tile_load<D, SWZ_K, BN>(k_rsrc, (uint32_t)(nb * BN) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane);
-        issue_tile_load<D, SWZ_V8, BN>(v_rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane);
+        issue_tile_load<D, SWZ_K, BN>(k_rsrc, (uint32_t)(nb * BNB) * k_sn, k_sn, lds0 + OFF_K + buf * KT, wave, k_lane);
+        issue_tile_load<D, SWZ_V8, BN>(v_rsrc, (uint32_t)(nb * BNB) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane);
     };
     // k_scale of a block: thread t < 128 fetches the scale of key t; converted to fp32 when stored to LDS
     const KScaleSource ks_src(p, b, hk, seqlen_k);
-    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t { return ks_src.load(nb * BN + (tid & (BN - 1))); };
+    auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t { return ks_src.load(nb * BNB + (tid & (BN - 1))); };
     auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
     // VBLK: fp32 channel scales of a key block; thread 128 + c fetches channel c
     const int vs_c = tid - 128;
@@ -109,7 +117,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + (vs_thread ? vs_c : 0));
     auto load_vs = [&](int nb) __attribute__((always_inline)) -> float {
         if (!VBLK) return 0.f;
-        const int row = p.vs_g == 1 ? nb : nb / p.vs_g;
+        const int row = p.vs_g == 1 ? nb : nb / p.vs_g;       // (VBLK: one block per step)
         return Vsg[(int64_t)row * p.vs_sblk];
     };
 
@@ -139,24 +147,23 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
     const uint32_t vs_wr = OFF_VS + 4 * (vs_thread ? vs_c : 0);
     const uint32_t vs_rd = OFF_VS + 16 * lh;                         // + 4 * (32*dt + 8*a4) per read
     const bool own_tile0 = wave < DT;                                // head_dim 64: waves 2 and 3 own no output tile
-    const int tail_keys = seqlen_k - (nb_total - 1) * BN;          // valid keys of the last block
-    // first block with a key hidden from the first row of this query block (never, without a causal mask)
-    const int diag_first = p.causal ? ((fold ? 0 : mb * kDecodeRows) + causal_off + 1) / BN : causal_end;
-    const int diag_begin = diag_first < 0 ? 0 : diag_first;
-    const int row_lim = p.causal ? (fold ? q_row % fold : q_row) + causal_off : 0x3fffffff;   // the lane's last visible key
+    // the last visible key of the first row of this query block, and of the lane's row
+    const int first_lim = p.causal ? (fold ? 0 : mb * kDecodeRows) + causal_off : 0x3fffffff;
+    const int row_lim = p.causal ? (fold ? q_row % fold : q_row) + causal_off : 0x3fffffff;
+    const bool blk_a = NBS == 1 || wave < 2;                          // this wave's keys belong to the first block of a step
 
     auto step = [&](auto buf_tag, int nb) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
         constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4, VSB = BUF * D * 4;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();                                   // tile nb has landed; the other buffer and the exchange areas are free
-        const bool more = nb + 1 < nb_end;
+        const bool more = nb + NBS < nb_end;
         uint32_t ks_next = 0;
         float vs_next = 0.f;
         if (more) {
-            issue_loads(nb + 1, BUF ^ 1);
-            if (tid < BN) ks_next = load_ks(nb + 1);
-            if (vs_thread) vs_next = load_vs(nb + 1);
+            issue_loads(nb + NBS, BUF ^ 1);
+            if (tid < BN) ks_next = load_ks(nb + NBS);
+            if (vs_thread) vs_next = load_vs(nb + NBS);
         }
         // -------- S^T of this wave's 32 keys, dequantise, partial row maximum
         v4i fr[KS];
@@ -183,11 +190,12 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
             }
         float x[16];
         float mx = -INFINITY;
-        // masked blocks (wave-uniform test): the ragged last block and the blocks the causal diagonal crosses
-        const bool tail = (nb == nb_total - 1 && tail_keys < BN) || nb >= diag_begin;
-        // keys of this lane with 8*a4 + b4 >= key_lim are hidden: past the end of the sequence or past the lane's row
-        const int last_key = row_lim - nb * BN < (nb == nb_total - 1 ? tail_keys : BN) - 1 ? row_lim - nb * BN
-                                                                                          : (nb == nb_total - 1 ? tail_keys : BN) - 1;
+        // masked steps (wave-uniform test): keys past the end of the range (the ragged last block; with two blocks per
+        // step, a second block that is not part of the range), or past the first row's position (the causal diagonal)
+        const int key0 = nb * BNB;
+        const bool tail = key0 + BN > key_end || key0 + BN - 1 > first_lim;
+        // keys of this lane with 8*a4 + b4 >= key_lim are hidden: past the end of the range or past the lane's row
+        const int last_key = (row_lim < key_end - 1 ? row_lim : key_end - 1) - key0;
         const int key_lim = last_key + 1 - 32 * wave - 4 * lh;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -199,13 +207,16 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
         mx = half_pair_max(mx);
         if (lh == 0) *(float*)(smem + xm_wr) = mx;
         __syncthreads();                                   // the four partial maxima are in LDS
-        mx = fmaxf(fmaxf(*(const float*)(smem + xm_rd), *(const float*)(smem + xm_rd + 128)),
-                   fmaxf(*(const float*)(smem + xm_rd + 256), *(const float*)(smem + xm_rd + 384)));
-        const float m_new = fmaxf(m_run, mx * qsc);
-        const float alpha = fast_exp2(m_run - m_new);
-        m_run = m_new;
-        // -------- P of this wave's keys, requantised; partial row sum
-        const float bias = (PROUND == 0 ? kLog2_127 : 0.f) - m_new;
+        // one block per step: alpha_b = 1 and m_a = m_b is the block's maximum; two blocks: the chain A, B
+        const float mx_a = fmaxf(*(const float*)(smem + xm_rd), *(const float*)(smem + xm_rd + 128));
+        const float mx_b = fmaxf(*(const float*)(smem + xm_rd + 256), *(const float*)(smem + xm_rd + 384));
+        const float m_a = fmaxf(m_run, (NBS == 1 ? fmaxf(mx_a, mx_b) : mx_a) * qsc);
+        const float alpha = fast_exp2(m_run - m_a);
+        const float m_b = NBS == 1 ? m_a : fmaxf(m_a, mx_b * qsc);
+        const float alpha_b = NBS == 1 ? 1.f : fast_exp2(m_a - m_b);
+        m_run = m_b;
+        // -------- P of this wave's keys, requantised in its block's frame; partial row sum
+        const float bias = (PROUND == 0 ? kLog2_127 : 0.f) - (blk_a ? m_a : m_b);
         float lsum = 0.f;
         v4i p8;
         {
@@ -244,16 +255,27 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
 #pragma unroll
         for (int j = 0; j < DTW; ++j) {
             if (j == 0 ? !own_tile0 : false) continue;
-            v16i acc = (v16i){0};
+            if (NBS == 1) {
+                v16i acc = (v16i){0};
 #pragma unroll
-            for (int st = 0; st < NST; ++st) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[j][st], pall[st], acc, 0, 0, 0);
+                for (int st = 0; st < NST; ++st) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[j][st], pall[st], acc, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                if (VBLK) o_acc[j][r] = fmaf(o_acc[j][r], alpha, (float)acc[r] * vsc[j][r >> 2][r & 3]);
-                else o_acc[j][r] = fmaf(o_acc[j][r], alpha, (float)acc[r]);
+                for (int r = 0; r < 16; ++r) {
+                    if (VBLK) o_acc[j][r] = fmaf(o_acc[j][r], alpha, (float)acc[r] * vsc[j][r >> 2][r & 3]);
+                    else o_acc[j][r] = fmaf(o_acc[j][r], alpha, (float)acc[r]);
+                }
+            } else {
+                v16i acc_a = (v16i){0}, acc_b = (v16i){0};
+#pragma unroll
+                for (int st = 0; st < NST / 2; ++st) acc_a = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[j][st], pall[st], acc_a, 0, 0, 0);
+#pragma unroll
+                for (int st = NST / 2; st < NST; ++st) acc_b = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[j][st], pall[st], acc_b, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o_acc[j][r] = fmaf(fmaf(o_acc[j][r], alpha, (float)acc_a[r]), alpha_b, (float)acc_b[r]);
             }
         }
-        l_run = fmaf(l_run, alpha, lsum);
+        if (NBS == 1) l_run = fmaf(l_run, alpha, lsum);
+        else l_run = blk_a ? fmaf(l_run, alpha, lsum) * alpha_b : fmaf(l_run * alpha, alpha_b, lsum);
         if (more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
         if (more && vs_thread) *(float*)(smem + vs_wr + (BUF ^ 1) * D * 4) = vs_next;
     };
@@ -265,9 +287,11 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_decode_full_int8_kernel(const
         int nb = nb_begin;
         while (true) {
             if (nb >= nb_end) break;
-            step(BoolTag<false>{}, nb++);
+            step(BoolTag<false>{}, nb);
+            nb += NBS;
             if (nb >= nb_end) break;
-            step(BoolTag<true>{}, nb++);
+            step(BoolTag<true>{}, nb);
+            nb += NBS;
         }
     }
 

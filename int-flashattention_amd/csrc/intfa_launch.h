@@ -36,6 +36,7 @@ INTFA_DECL_LAUNCH(launch_full_int8_vblk64_d64);   // V scale rows of 64 keys (tw
 INTFA_DECL_LAUNCH(launch_full_int8_vblk64_d128);
 INTFA_DECL_LAUNCH(launch_decode_full_int8_d64);    // few query rows per head: the waves of a workgroup share the keys
 INTFA_DECL_LAUNCH(launch_decode_full_int8_d128);
+INTFA_DECL_LAUNCH(launch_decode_full_int8_d256);
 INTFA_DECL_LAUNCH(launch_decode_half_int8_d64);     // (intfa_fwd_decode_f16pv.h)
 INTFA_DECL_LAUNCH(launch_decode_half_int8_d128);
 INTFA_DECL_LAUNCH(launch_decode_fp16_d64);
