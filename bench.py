@@ -83,6 +83,8 @@ WORKLOADS = {
     # the same decode shape for the two variants with a 16-bit V cache (int8 or 16-bit K cache)
     "half_int8_decode_B32_H32_Nq1_Nk4096_d128": dict(variant="half", B=32, H=32, N=1, Nk=4096, D=128, causal=False, splits=1),
     "fp16_decode_B32_H32_Nq1_Nk4096_d128": dict(variant="fp", B=32, H=32, N=1, Nk=4096, D=128, causal=False, splits=1),
+    "half_int8_decode_B32_H32_Nq1_Nk4096_d256": dict(variant="half", B=32, H=32, N=1, Nk=4096, D=256, causal=False, splits=1),
+    "fp16_decode_B32_H32_Nq1_Nk4096_d256": dict(variant="fp", B=32, H=32, N=1, Nk=4096, D=256, causal=False, splits=1),
     # the input quantisers (HBM-bound): Q/K per token, V per (batch, head)
     "quant_pertoken_B4_H32_N4096_d128": dict(variant="quant_token", B=4, H=32, N=4096, D=128, causal=False, splits=1),
     "quant_pertensor_B4_H32_N4096_d128": dict(variant="quant_tensor", B=4, H=32, N=4096, D=128, causal=False, splits=1),

@@ -143,8 +143,8 @@ typedef struct intfa_fwd_params {
                                  K/V group one after the other (decoding with grouped heads described as heads = heads_kv,
                                  seqlen = group * positions, see heads_kv): row r is position r % causal_rows for the causal
                                  mask.  Only with causal and the shapes of the decode kernels: seqlen <= 64 and
-                                 head_dim <= 128 (any variant; not with v_scale_block = 64), or head_dim 256 in the
-                                 full-int8 variant with v_scale_block = 0.  seqlen must be a multiple of it. */
+                                 head_dim <= 128 (not with v_scale_block = 64) or head_dim 256 (not with blocked V
+                                 scales), any variant.  seqlen must be a multiple of it. */
     int32_t reserved1;        /* set to 0 */
 } intfa_fwd_params;
 

@@ -152,12 +152,11 @@ int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t str
 
 // Few query rows per head (decoding against a cache): the pass runs a kernel whose waves share the keys of a block
 // instead of each taking 32 query rows (intfa_fwd_decode.h, intfa_fwd_decode_f16pv.h).
-// Head_dim 256: the full-int8 variant with one V scale per (batch, head); its other forms and the 16-bit V caches of the
-// other variants (their tiles of a step do not fit the LDS twice) stay with the general kernels.
+// (Head_dim 256 of the full-int8 variant with blocked V scales stays with the general kernel.)
 constexpr int kDecodeMaxRows = 2 * kDecodeRows;
 bool decode_shaped(int variant, int seqlen, int head_dim, bool blocked_v_scales) {
     if (seqlen > kDecodeMaxRows) return false;
-    return head_dim <= 128 || (head_dim == 256 && variant == INTFA_VARIANT_FULL_INT8 && !blocked_v_scales);
+    return head_dim <= 128 || !(variant == INTFA_VARIANT_FULL_INT8 && blocked_v_scales);
 }
 
 int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dump_s, hipStream_t stream) {
@@ -180,9 +179,11 @@ int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dum
         } else if (variant == INTFA_VARIANT_HALF_INT8) {
             if (d == 64) return launch_decode_half_int8_d64(kp, sel, stream);
             if (d == 128) return launch_decode_half_int8_d128(kp, sel, stream);
+            if (d == 256) return launch_decode_half_int8_d256(kp, sel, stream);
         } else {
             if (d == 64) return launch_decode_fp16_d64(kp, sel, stream);
             if (d == 128) return launch_decode_fp16_d128(kp, sel, stream);
+            if (d == 256) return launch_decode_fp16_d256(kp, sel, stream);
         }
     } else if (vblk) {
         if (d == 64) return launch_full_int8_vblk_d64(kp, sel, stream);

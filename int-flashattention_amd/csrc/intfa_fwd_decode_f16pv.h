@@ -14,6 +14,9 @@
 // Every block is evaluated with the same maximum, the same P and the same order of MFMA steps as in the general kernel;
 // only the row sums are added in another order (per wave, joined in the epilogue).  K/V tiles of a step are
 // double-buffered in LDS and the whole next step is requested at the start of a step.
+// Head_dim 256: 128 keys of 16-bit V (and K) do not fit the LDS twice, so a step is ONE 64-key block there: waves 0 and 1
+// compute S^T and P for its two 32-key sub-tiles, waves 2 and 3 only wait at the barriers in that phase (the pass is
+// bound by the stream of K and V, not by the arithmetic), and every wave owns two 32-column output tiles.
 #pragma once
 #include "intfa_device.h"
 #include "intfa_launch.h"
@@ -25,21 +28,25 @@ namespace intfa {
 // when !QK_INT8): 0 fp16, 1 bf16.  The causal mask is a run-time switch here (p.causal).
 template <bool QK_INT8, int D, int IO_DT, bool SPLIT>
 __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_kernel(const KParams p) {
-    static_assert(D == 64 || D == 128, "head_dim 256 keeps its eight-wave kernel");
+    static_assert(D == 64 || D == 128 || D == 256, "head dims 64, 128 and 256");
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int BNB = kBlockN16;                    // key block of the arithmetic
-    constexpr int BN = 2 * BNB;                       // keys per step: one 32-key sub-tile per wave
+    constexpr int NBS = D <= 128 ? 2 : 1;             // key blocks per step
+    constexpr int BN = NBS * BNB;                     // keys per step
+    constexpr int QKW = BN / 32;                      // waves with a 32-key sub-tile of S^T (all four, or waves 0 and 1)
     constexpr int NG = BN / 16;                       // 16-key MFMA steps of P V per step (two per wave's sub-tile)
     constexpr int QB = QK_INT8 ? 1 : 2;               // bytes per Q/K element
     constexpr int KROW = D * QB, VROW = D * 2;
     constexpr int KS = KROW / 32;                     // MFMA k-steps of S^T
-    constexpr int DT = D / 32;                        // 32-wide output tiles; wave w owns tile w (head_dim 64: waves 0, 1)
+    constexpr int DT = D / 32;                        // 32-wide output tiles; wave w owns tiles w, w + 4 (head_dim 64: waves 0, 1)
+    constexpr int DTW = (DT + 3) / 4;                 // output tiles per wave
     constexpr int KT = BN * KROW, VT = BN * VROW;
     constexpr int KCH = KROW / 16, VCH = VROW / 16;
     // LDS map (bytes)
     constexpr int OFF_KS = 0;                             // two fp32 k_scale vectors
     constexpr int OFF_XM = 2 * BN * 4;                    // 4 waves x 32 rows fp32: partial row maxima / row sums
     constexpr int OFF_XP = OFF_XM + 4 * 32 * 4;           // NG operands of 64 lanes x 16 bytes: the waves' 16-bit P
+    static_assert(QKW == 4 || QKW == 2, "a step is four or two 32-key sub-tiles");
     constexpr int OFF_K = OFF_XP + NG * 1024;
     constexpr int OFF_V = OFF_K + 2 * KT;
     constexpr int LDS_BYTES = OFF_V + 2 * VT;
@@ -87,9 +94,11 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
     const float qsc = QK_INT8 ? load_q_scale_log2(p, b, h, q_ld) : p.qk_scale_log2;
 
     float m_run = -INFINITY, l_run = 0.f;        // l_run: this wave's keys only
-    v16f o_acc;
+    v16f o_acc[DTW];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o_acc[r] = 0.f;
+    for (int j = 0; j < DTW; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[j][r] = 0.f;
 
     // ---- global -> LDS copies (asynchronous, straight into LDS; the four waves split the instructions)
     const char* Kg = p.k + b * p.k_sb + hk * p.k_sh;
@@ -122,9 +131,14 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
     const int v_row0 = 4 * lh + (s16 >> 2);           // + 8 for the second load, + 16 per MFMA step
     const int v_swz = swz_v16<VROW>(v_row0) & (VCH - 1);
     const bool own_tile = wave < DT;                  // head_dim 64: waves 2 and 3 own no output tile
-    const int dt_own = own_tile ? wave : 0;
-    const int v_c = 4 * dt_own + 2 * (g16 & 1) + ((s16 & 3) >> 1);
-    const uint32_t v_rd = OFF_V + v_row0 * VROW + ((v_c ^ v_swz) << 4) + 8 * (s16 & 1);
+    const bool qk_wave = wave < QKW;                  // this wave computes a sub-tile of S^T and its P
+    uint32_t v_rd[DTW];
+#pragma unroll
+    for (int j = 0; j < DTW; ++j) {
+        const int dt = own_tile ? wave + 4 * j : 0;
+        const int v_c = 4 * dt + 2 * (g16 & 1) + ((s16 & 3) >> 1);
+        v_rd[j] = OFF_V + v_row0 * VROW + ((v_c ^ v_swz) << 4) + 8 * (s16 & 1);
+    }
     const uint32_t ks_rd = OFF_KS + 4 * (32 * wave) + 16 * lh;       // + 4 * 8*a4 per read
     const uint32_t ks_wr = OFF_KS + 4 * (tid & (BN - 1));
     const uint32_t xm_wr = OFF_XM + 4 * (32 * wave + lq);
@@ -134,7 +148,7 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
     // the smallest and this lane's own last visible key
     const int first_lim = p.causal ? (fold ? 0 : mb * kDecodeRows) + causal_off : 0x3fffffff;
     const int row_lim = p.causal ? (fold ? q_row % fold : q_row) + causal_off : 0x3fffffff;
-    const bool blk_a = wave < 2;                      // this wave's keys belong to the first block of a step
+    const bool blk_a = NBS == 1 || wave < 2;          // this wave's keys belong to the first block of a step
 
     auto mfma16 = [&](v4i a, v4i bb, v16f c) __attribute__((always_inline)) -> v16f {
         if (IO_DT == 0) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, bb), c, 0, 0, 0);
@@ -147,38 +161,42 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
         constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();                                   // the tiles have landed; the other buffer and the exchange areas are free
-        const bool more = nb + 2 < nb_end;
+        const bool more = nb + NBS < nb_end;
         uint32_t ks_next = 0;
         if (more) {
-            issue_loads(nb + 2, BUF ^ 1);
-            ks_next = load_ks(nb + 2);
+            issue_loads(nb + NBS, BUF ^ 1);
+            ks_next = load_ks(nb + NBS);
         }
         // -------- S^T of this wave's 32 keys, dequantise, partial row maximum
         v4i fr[KS];
         v4f kk[4];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) fr[ks] = *(const v4i*)(smem + k_rd[ks] + KB);
-        if (QK_INT8) {
-#pragma unroll
-            for (int a4 = 0; a4 < 4; ++a4) kk[a4] = *(const v4f*)(smem + ks_rd + SB + 4 * 8 * a4);
-        }
         v16i si = (v16i){0};
         v16f sf = (v16f){0};
+        if (qk_wave) {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            if (QK_INT8) si = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[ks], qreg[ks], si, 0, 0, 0);
-            else sf = mfma16(fr[ks], qreg[ks], sf);
+            for (int ks = 0; ks < KS; ++ks) fr[ks] = *(const v4i*)(smem + k_rd[ks] + KB);
+            if (QK_INT8) {
+#pragma unroll
+                for (int a4 = 0; a4 < 4; ++a4) kk[a4] = *(const v4f*)(smem + ks_rd + SB + 4 * 8 * a4);
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                if (QK_INT8) si = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[ks], qreg[ks], si, 0, 0, 0);
+                else sf = mfma16(fr[ks], qreg[ks], sf);
+            }
         }
-        // V fragments of this wave's output tile (all keys of the step) travel during the softmax
-        v4i vf[NG];
+        // V fragments of this wave's output tiles (all keys of the step) travel during the softmax
+        v4i vf[DTW][NG];
         if (own_tile) {
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                const uint32_t a0 = v_rd + VB + 16 * g * VROW;
-                const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)INTFA_LDS(smem + a0));
-                const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)INTFA_LDS(smem + a0 + 8 * VROW));
-                vf[g] = (v4i){__builtin_bit_cast(v2i, lo)[0], __builtin_bit_cast(v2i, lo)[1], __builtin_bit_cast(v2i, hi)[0], __builtin_bit_cast(v2i, hi)[1]};
-            }
+            for (int j = 0; j < DTW; ++j)
+#pragma unroll
+                for (int g = 0; g < NG; ++g) {
+                    const uint32_t a0 = v_rd[j] + VB + 16 * g * VROW;
+                    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)INTFA_LDS(smem + a0));
+                    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)INTFA_LDS(smem + a0 + 8 * VROW));
+                    vf[j][g] = (v4i){__builtin_bit_cast(v2i, lo)[0], __builtin_bit_cast(v2i, lo)[1], __builtin_bit_cast(v2i, hi)[0], __builtin_bit_cast(v2i, hi)[1]};
+                }
         }
         const int key0 = nb * BNB;
         // masked steps (wave-uniform test): keys past the end of the range, or past the first row's position
@@ -188,27 +206,32 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
         const int key_lim = last_key + 1 - 32 * wave - 4 * lh;
         float x[16];
         float mx = -INFINITY;
+        if (qk_wave) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            float v = QK_INT8 ? (float)si[r] * kk[r >> 2][r & 3] : sf[r];
-            if (tail && 8 * (r >> 2) + (r & 3) >= key_lim) v = -INFINITY;
-            x[r] = v;
-            mx = fmaxf(mx, v);
+            for (int r = 0; r < 16; ++r) {
+                float v = QK_INT8 ? (float)si[r] * kk[r >> 2][r & 3] : sf[r];
+                if (tail && 8 * (r >> 2) + (r & 3) >= key_lim) v = -INFINITY;
+                x[r] = v;
+                mx = fmaxf(mx, v);
+            }
+            mx = half_pair_max(mx);
+            if (lh == 0) *(float*)(smem + xm_wr) = mx;
         }
-        mx = half_pair_max(mx);
-        if (lh == 0) *(float*)(smem + xm_wr) = mx;
-        __syncthreads();                                   // the four partial maxima are in LDS
+        __syncthreads();                                   // the partial maxima are in LDS
         const float mx_a = fmaxf(*(const float*)(smem + xm_rd), *(const float*)(smem + xm_rd + 128));
-        const float mx_b = fmaxf(*(const float*)(smem + xm_rd + 256), *(const float*)(smem + xm_rd + 384));
         const float m_a = fmaxf(m_run, mx_a * qsc);
         const float alpha_a = fast_exp2(m_run - m_a);
-        const float m_b = fmaxf(m_a, mx_b * qsc);
-        const float alpha_b = fast_exp2(m_a - m_b);
+        float m_b = m_a, alpha_b = 1.f;                    // one block per step: no second factor
+        if (NBS == 2) {
+            const float mx_b = fmaxf(*(const float*)(smem + xm_rd + 256), *(const float*)(smem + xm_rd + 384));
+            m_b = fmaxf(m_a, mx_b * qsc);
+            alpha_b = fast_exp2(m_a - m_b);
+        }
         m_run = m_b;
         // -------- P of this wave's keys in 16 bits; partial row sum
         const float m_own = blk_a ? m_a : m_b;
         float lsum = 0.f;
-        {
+        if (qk_wave) {
             float e[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -220,22 +243,28 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
                 *(v4i*)(smem + xp_wr + 1024 * u) = IO_DT == 0 ? __builtin_bit_cast(v4i, pack_p_f16(e + 8 * u))
                                                               : __builtin_bit_cast(v4i, pack_p_bf16(e + 8 * u));
         }
-        __syncthreads();                                   // the eight P operands are in LDS
+        __syncthreads();                                   // the P operands are in LDS
         // -------- this wave's output columns: O^T[d, q] = (O^T alpha_A + V_A^T P_A^T) alpha_B + V_B^T P_B^T
         if (own_tile) {
             v4i pall[NG];
 #pragma unroll
             for (int g = 0; g < NG; ++g) pall[g] = *(const v4i*)(smem + xp_rd + 1024 * g);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o_acc[r] *= alpha_a;
+            for (int j = 0; j < DTW; ++j) {
 #pragma unroll
-            for (int g = 0; g < NG / 2; ++g) o_acc = mfma16(vf[g], pall[g], o_acc);
+                for (int r = 0; r < 16; ++r) o_acc[j][r] *= alpha_a;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o_acc[r] *= alpha_b;
+                for (int g = 0; g < NG / NBS; ++g) o_acc[j] = mfma16(vf[j][g], pall[g], o_acc[j]);
+                if (NBS == 2) {
 #pragma unroll
-            for (int g = NG / 2; g < NG; ++g) o_acc = mfma16(vf[g], pall[g], o_acc);
+                    for (int r = 0; r < 16; ++r) o_acc[j][r] *= alpha_b;
+#pragma unroll
+                    for (int g = NG / 2; g < NG; ++g) o_acc[j] = mfma16(vf[j][g], pall[g], o_acc[j]);
+                }
+            }
         }
-        l_run = blk_a ? fmaf(l_run, alpha_a, lsum) * alpha_b : fmaf(l_run * alpha_a, alpha_b, lsum);
+        if (NBS == 1) l_run = fmaf(l_run, alpha_a, lsum);
+        else l_run = blk_a ? fmaf(l_run, alpha_a, lsum) * alpha_b : fmaf(l_run * alpha_a, alpha_b, lsum);
         if (QK_INT8 && more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
     };
 
@@ -248,10 +277,10 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
         int nb = nb_begin;
         while (true) {
             step(BoolTag<false>{}, nb);
-            nb += 2;
+            nb += NBS;
             if (nb >= nb_end) break;
             step(BoolTag<true>{}, nb);
-            nb += 2;
+            nb += NBS;
             if (nb >= nb_end) break;
         }
     }
@@ -274,12 +303,14 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
         float* op = p.o_part + row * D;
         if (own_tile) {
 #pragma unroll
-            for (int a4 = 0; a4 < 4; ++a4) {
-                v4f o;
+            for (int j = 0; j < DTW; ++j)
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[4 * a4 + b4] * inv : 0.f;
-                *(v4f*)(op + 32 * wave + 8 * a4 + 4 * lh) = o;
-            }
+                for (int a4 = 0; a4 < 4; ++a4) {
+                    v4f o;
+#pragma unroll
+                    for (int b4 = 0; b4 < 4; ++b4) o[b4] = seen ? o_acc[j][4 * a4 + b4] * inv : 0.f;
+                    *(v4f*)(op + 32 * (wave + 4 * j) + 8 * a4 + 4 * lh) = o;
+                }
         }
         if (wave == 0 && lh == 0) p.lse_part[row] = lse;
         return;
@@ -287,20 +318,22 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
     char* orow = p.out + b * p.o_sb + h * p.o_sh + (int64_t)q_row * p.o_sn;
     if (own_tile) {
 #pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) {
-            const int d0 = 32 * wave + 8 * a4 + 4 * lh;
-            if (IO_DT == 0) {
-                v4h o;
+        for (int j = 0; j < DTW; ++j)
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(seen ? o_acc[4 * a4 + b4] * inv : 0.f);
-                *(v4h*)(orow + d0 * 2) = o;
-            } else {
-                v4s o;
+            for (int a4 = 0; a4 < 4; ++a4) {
+                const int d0 = 32 * (wave + 4 * j) + 8 * a4 + 4 * lh;
+                if (IO_DT == 0) {
+                    v4h o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(seen ? o_acc[4 * a4 + b4] * inv : 0.f);
-                *(v4s*)(orow + d0 * 2) = o;
+                    for (int b4 = 0; b4 < 4; ++b4) o[b4] = (_Float16)(seen ? o_acc[j][4 * a4 + b4] * inv : 0.f);
+                    *(v4h*)(orow + d0 * 2) = o;
+                } else {
+                    v4s o;
+#pragma unroll
+                    for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(seen ? o_acc[j][4 * a4 + b4] * inv : 0.f);
+                    *(v4s*)(orow + d0 * 2) = o;
+                }
             }
-        }
     }
     if (p.lse != nullptr && wave == 0 && lh == 0) p.lse[((int64_t)b * p.heads + h) * p.seqlen + q_row] = lse;
 #endif  // __HIP_DEVICE_COMPILE__

@@ -1,0 +1,3 @@
+#define INTFA_INST_D 256
+#define INTFA_INST_QK_INT8 1
+#include "intfa_inst_decode_f16pv.inc"

@@ -39,8 +39,10 @@ INTFA_DECL_LAUNCH(launch_decode_full_int8_d128);
 INTFA_DECL_LAUNCH(launch_decode_full_int8_d256);
 INTFA_DECL_LAUNCH(launch_decode_half_int8_d64);     // (intfa_fwd_decode_f16pv.h)
 INTFA_DECL_LAUNCH(launch_decode_half_int8_d128);
+INTFA_DECL_LAUNCH(launch_decode_half_int8_d256);
 INTFA_DECL_LAUNCH(launch_decode_fp16_d64);
 INTFA_DECL_LAUNCH(launch_decode_fp16_d128);
+INTFA_DECL_LAUNCH(launch_decode_fp16_d256);
 INTFA_DECL_LAUNCH(launch_half_int8_d64);
 INTFA_DECL_LAUNCH(launch_half_int8_d128);
 INTFA_DECL_LAUNCH(launch_half_int8_d256);

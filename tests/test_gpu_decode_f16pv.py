@@ -1,5 +1,5 @@
 """GPU parity of the decode-shaped half-int8 and fp16/bf16 forward (few query rows per head against a long key/value
-cache, head_dim <= 128): the kernel whose four waves share two 64-key blocks per step, through the C ABI, against the
+cache): the kernel whose four waves share two 64-key blocks per step (one at head_dim 256), through the C ABI, against the
 CPU oracle (flash_atten_int8.py:9-66, flash_atten_fp.py:9-60 restated with separate query and key lengths) at the
 kernel's 64-key block.
 
@@ -80,6 +80,15 @@ SHAPES = [
     (1, 2, 2, 64, 64, 128, True),        # square: row i sees keys 0 .. i
     (1, 2, 2, 40, 20, 128, True),        # more new tokens than keys: rows above the first key see nothing
     (1, 1, 1, 3, 4096, 128, False),
+    # head_dim 256: one 64-key block per step, two output tiles per wave
+    (2, 4, 4, 1, 1000, 256, False),
+    (1, 8, 2, 1, 2048, 256, False),
+    (1, 2, 2, 33, 577, 256, False),
+    (1, 2, 1, 7, 50, 256, False),
+    (1, 2, 2, 64, 64, 256, True),
+    (2, 2, 2, 9, 1000, 256, True),
+    (1, 8, 2, 6, 333, 256, True),
+    (1, 2, 2, 40, 20, 256, True),
 ]
 
 
@@ -102,7 +111,7 @@ def test_decode_matches_oracle(B, H, H_kv, Nq, Nk, D, causal, variant, dtype):
 
 
 @pytest.mark.parametrize("variant", ["half", "fp"])
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [64, 128, 256])
 @pytest.mark.parametrize("causal", [False, True])
 def test_decode_kernel_agrees_with_the_general_kernel(variant, D, causal):
     """65 query rows run the general kernel, 64 of them alone the decode kernel: same block maxima, same 16-bit P and the
@@ -119,12 +128,12 @@ def test_decode_kernel_agrees_with_the_general_kernel(variant, D, causal):
 
 
 @pytest.mark.parametrize("variant", ["half", "fp"])
+@pytest.mark.parametrize("D", [128, 256])
 @pytest.mark.parametrize("Nq,Nk,causal,splits", [(3, 2000, False, 2), (3, 2000, False, 5), (1, 4100, False, "auto"), (17, 1000, True, 3),
                                                  (40, 333, True, 4)])
-def test_decode_split_kv_equals_single_pass(variant, Nq, Nk, causal, splits):
+def test_decode_split_kv_equals_single_pass(variant, D, Nq, Nk, causal, splits):
     """The split evaluation is the same sum in another order, except that P is cast to 16 bits relative to another running
     maximum: it agrees with the single pass to a fraction of an output ulp in the mean, and its LSE to fp32 rounding."""
-    D = 128
     q, k, v = inputs(2, 4, 4, Nq, Nk, D, seed=3200 + Nq)
     sm = D ** -0.5
     o1, l1 = run(variant, q, k, v, causal, sm, return_lse=True)
@@ -137,11 +146,12 @@ def test_decode_split_kv_equals_single_pass(variant, Nq, Nk, causal, splits):
 
 
 @pytest.mark.parametrize("variant", ["half", "fp"])
+@pytest.mark.parametrize("D", [128, 256])
 @pytest.mark.parametrize("causal", [False, True])
-def test_decode_per_batch_cache_lengths(variant, causal):
+def test_decode_per_batch_cache_lengths(variant, D, causal):
     """seqlens_k: every batch entry comes out as a call on that entry with the cache cut to its length (an empty entry
     gives zeros)."""
-    B, H, Nq, Nk, D = 4, 2, 5, 600, 128
+    B, H, Nq, Nk = 4, 2, 5, 600
     lens = [600, 1, 333, 0]
     q, k, v = inputs(B, H, H, Nq, Nk, D, seed=3300)
     sm = D ** -0.5
