@@ -77,6 +77,14 @@ struct KParams {
     float qk_scale_log2;                   // sm_scale * log2(e)
 };
 
+// The kernel's own argument block as the epilogues re-read it: the pointer keeps the constant address space, so its
+// fields arrive through scalar loads (a generic pointer would make them vector loads that a vmcnt wait has to cover).
+typedef const __attribute__((address_space(4))) KParams* KernargPtr;
+__device__ __forceinline__ KernargPtr kernarg_block() {
+    KernargPtr pe = (KernargPtr)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(pe));       // opaque: the fields are loaded where they are used, not held since the prologue
+    return pe;
+}
 __device__ __forceinline__ float load_scale(const char* base, int64_t idx, int dtype) {
     if (dtype == 0) return (float)((const _Float16*)base)[idx];
     if (dtype == 1) return __builtin_bit_cast(float, ((uint32_t)((const uint16_t*)base)[idx]) << 16);

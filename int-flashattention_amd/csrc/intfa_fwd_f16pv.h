@@ -325,8 +325,7 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
     }
 
     // ---- epilogue
-    const KParams* pe = (const KParams*)__builtin_amdgcn_kernarg_segment_ptr();
-    asm volatile("" : "+s"(pe));
+    const KernargPtr pe = kernarg_block();
     const int e_heads = pe->heads, e_seqlen = pe->seqlen;
     const int eb = head / e_heads, eh = head % e_heads;
     const float l_tot = half_pair_sum(l_run);

@@ -509,8 +509,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
 
     // ---- epilogue.  Everything it needs from the parameter block is (re)loaded here, behind an opaque copy of the
     // kernel-argument pointer, so that these values do not occupy scalar registers during the main loop.
-    const KParams* pe = (const KParams*)__builtin_amdgcn_kernarg_segment_ptr();
-    asm volatile("" : "+s"(pe));
+    const KernargPtr pe = kernarg_block();
     const int e_heads = pe->heads, e_seqlen = pe->seqlen;
     const int eb = head / e_heads, eh = head % e_heads;
     const float l_tot = half_pair_sum(l_run);          // in units of 1/127 when PROUND == 0

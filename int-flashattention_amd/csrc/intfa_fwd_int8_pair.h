@@ -337,8 +337,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
     }
 
     // ---- epilogue
-    const KParams* pe = (const KParams*)__builtin_amdgcn_kernarg_segment_ptr();
-    asm volatile("" : "+s"(pe));
+    const KernargPtr pe = kernarg_block();
     const int e_heads = pe->heads, e_seqlen = pe->seqlen;
     const int eb = head / e_heads, eh = head % e_heads;
     // row sum: this wave's keys plus the partner's (the last block's barriers lie between the last use of the exchange
