@@ -50,6 +50,13 @@ constexpr float kMagicF = 12582912.f;
 // directly to an element of an ext_vector (acc[r]) reads element 0 whatever r is (clang 22 of ROCm 7.2).
 __device__ __forceinline__ float as_f32(int x) { return __builtin_bit_cast(float, x); }
 
+// floor(n / d) for 0 <= n < 2^31 and a divisor d fixed per launch: (n * m) >> s with s = 31 + ceil(log2 d) and
+// m = ceil(2^s / d) < 2^32 computed on the host (Granlund & Montgomery, "Division by invariant integers using
+// multiplication").  For a wave-uniform n that is three scalar instructions; a run-time integer division expands to some
+// forty dependent vector instructions, and the mapping of a workgroup to its work needs a dozen of them.
+struct FastDiv { uint32_t m, s; };
+__host__ __device__ __forceinline__ int fast_div(int n, FastDiv d) { return (int)(((uint64_t)(uint32_t)n * d.m) >> d.s); }
+
 // Kernel-side parameter block (byte strides, resolved pointers).
 struct KParams {
     const char* q; const char* k; const char* v; char* out;
@@ -75,6 +82,11 @@ struct KParams {
     int32_t vs_sub;                        // blocked V scales: 2 when a scale row covers 64 keys, half of the 128-key block
     int32_t causal_rows;                   // decode kernel: query positions per folded query head (0 = the row is the position)
     float qk_scale_log2;                   // sm_scale * log2(e)
+    // workgroup -> work mapping of this launch (set by finish_mapping() in intfa_launch.h from the grid size)
+    int32_t per_head;                      // workgroups per query head
+    int32_t heads_kv;                      // heads / kv_group
+    int32_t xcd_deal;                      // 1: the K/V heads divide evenly among the 8 XCDs
+    FastDiv d_per_kv, d_heads_kv, d_per_head, d_n_split, d_heads, d_kv_group;
 };
 
 // The kernel's own argument block as the epilogues re-read it: the pointer keeps the constant address space, so its
@@ -98,23 +110,25 @@ __device__ __forceinline__ float load_scale(const char* base, int64_t idx, int d
 // the 8 XCDs, each with its own L2: every XCD gets whole K/V heads, so the K/V tiles of a head are re-read from one L2.
 // With grouped K/V heads (kv_group query heads share one K/V head) the unit dealt to an XCD is the K/V head: all query
 // heads of a group run on the XCD whose L2 holds their K/V.
-struct WorkgroupJob { int head, rem; };
-__device__ __forceinline__ WorkgroupJob deal_workgroup(const KParams& p, int bid, int per_head) {
+// (All divisors are fixed per launch: fast_div.)
+struct WorkgroupJob { int b, h, hk, rem; };      // batch entry, query head, K/V head, index among the head's workgroups
+__device__ __forceinline__ WorkgroupJob deal_workgroup(const KParams& p, int bid) {
     const int kv_group = p.kv_group;
+    const int per_head = p.per_head;
     const int per_kv = per_head * kv_group;              // workgroups per K/V head
-    const int n_kv = p.batch * p.heads / kv_group;
     int kv_lin, r;
-    if ((n_kv & 7) == 0) {
+    if (p.xcd_deal) {
         const int xcd = bid & 7, slot = bid >> 3;
-        kv_lin = (slot / per_kv) * 8 + xcd;
-        r = slot % per_kv;
+        const int q = fast_div(slot, p.d_per_kv);
+        kv_lin = q * 8 + xcd;
+        r = slot - q * per_kv;
     } else {
-        kv_lin = bid / per_kv;
-        r = bid % per_kv;
+        kv_lin = fast_div(bid, p.d_per_kv);
+        r = bid - kv_lin * per_kv;
     }
-    const int heads_kv = p.heads / kv_group;
-    const int bb = kv_lin / heads_kv, hk = kv_lin % heads_kv;
-    return {bb * p.heads + hk * kv_group + r / per_head, r % per_head};
+    const int bb = fast_div(kv_lin, p.d_heads_kv), hk = kv_lin - bb * p.heads_kv;
+    const int hq = fast_div(r, p.d_per_head);            // query head inside the group
+    return {bb, hk * kv_group + hq, hk, r - hq * per_head};
 }
 
 // Number of keys of batch entry b: one length for all, or per batch (a cache filled to different lengths), clamped to

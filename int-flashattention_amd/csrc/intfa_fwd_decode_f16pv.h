@@ -61,13 +61,11 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
     // ---- block -> (head, 32-row query block, split)
     const int n_mblk = (p.seqlen + kDecodeRows - 1) / kDecodeRows;
     const int n_split = SPLIT ? p.num_splits : 1;
-    const int per_head = n_mblk * n_split;
-    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x, per_head);
-    const int rem = wg.rem, head = wg.head;
-    const int kv_group = p.kv_group;
-    const int mb = rem / n_split, split = rem % n_split;
-    const int b = head / p.heads, h = head % p.heads;
-    const int hk = h / kv_group;
+    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x);
+    const int rem = wg.rem, head = wg.b * p.heads + wg.h;
+    const int mb = fast_div(rem, p.d_n_split), split = rem - mb * n_split;
+    const int b = wg.b, h = wg.h;
+    const int hk = wg.hk;
 
     const int seqlen_k = keys_of_batch(p, b);
     // causal: the row at position i sees keys 0 .. i + causal_off (mask aligned to the bottom right corner)

@@ -66,21 +66,19 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
     // Causal single-pass launches pair query block i with query block n-1-i in one workgroup (heavy one first): every
     // workgroup then walks the same number of key blocks and the launch has no tail of light workgroups.
     const bool pair = CAUSAL && !SPLIT && p.pair_mblocks != 0;
-    const int per_head = (pair ? n_mblk / 2 : n_mblk * n_split) * NHALF;
-    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x, per_head);
-    const int rem = wg.rem, head = wg.head;
-    const int kv_group = p.kv_group;
+    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x);
+    const int rem = wg.rem, head = wg.b * p.heads + wg.h;
     const int half = rem % NHALF;                // column half of this workgroup (0 when the columns are not split)
-    const int mb_idx = (rem / NHALF) / n_split;
-    const int split = (rem / NHALF) % n_split;
+    const int mb_idx = fast_div(rem / NHALF, p.d_n_split);
+    const int split = rem / NHALF - mb_idx * n_split;
     const int njobs = pair ? 2 : 1;
 #pragma clang loop unroll(disable)
     for (int job = 0; job < njobs; ++job) {
     if (job) __syncthreads();                    // every wave is done with the LDS tiles of the first query block
     int mb = mb_idx;
     if (CAUSAL) mb = (pair && job) ? mb_idx : n_mblk - 1 - mb_idx;     // heaviest query blocks first
-    const int b = head / p.heads, h = head % p.heads;
-    const int hk = h / kv_group;                     // K/V head of this query head
+    const int b = wg.b, h = wg.h;
+    const int hk = wg.hk;                     // K/V head of this query head
     // ragged sequence lengths are handled as in the full-int8 kernel (zero-filled copies, masked last block, rows past
     // the end computed on clamped inputs and not stored)
     const int seqlen_k = keys_of_batch(p, b);
@@ -327,7 +325,7 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
     // ---- epilogue
     const KernargPtr pe = kernarg_block();
     const int e_heads = pe->heads, e_seqlen = pe->seqlen;
-    const int eb = head / e_heads, eh = head % e_heads;
+    const int eb = fast_div(head, pe->d_heads), eh = head - eb * e_heads;
     const float l_tot = half_pair_sum(l_run);
     // (no key at all - an empty cache entry - gives zeros and lse = -inf instead of 0 / 0)
     const bool any_key = nb_begin < nb_end && m_run > -INFINITY;      // (a causal row above the first key sees nothing)

@@ -66,20 +66,18 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     // Causal single-pass launches pair query block i with query block n-1-i in one workgroup (heavy one first): every
     // workgroup then walks the same number of key blocks and the launch has no tail of light workgroups.
     const bool pair = CAUSAL && !SPLIT && p.pair_mblocks != 0;
-    const int per_head = pair ? n_mblk / 2 : n_mblk * n_split;
-    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x, per_head);
-    const int head = wg.head, rem = wg.rem;
-    const int kv_group = p.kv_group;
-    const int mb_idx = rem / n_split;
-    const int split = rem % n_split;
+    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x);
+    const int rem = wg.rem, head = wg.b * p.heads + wg.h;
+    const int mb_idx = fast_div(rem, p.d_n_split);
+    const int split = rem - mb_idx * n_split;
     const int njobs = pair ? 2 : 1;
 #pragma clang loop unroll(disable)
     for (int job = 0; job < njobs; ++job) {
     if (job) __syncthreads();                    // every wave is done with the LDS tiles of the first query block
     int mb = mb_idx;
     if (CAUSAL) mb = (pair && job) ? mb_idx : n_mblk - 1 - mb_idx;     // heaviest query blocks first
-    const int b = head / p.heads, h = head % p.heads;
-    const int hk = h / kv_group;                     // K/V head of this query head
+    const int b = wg.b, h = wg.h;
+    const int hk = wg.hk;                     // K/V head of this query head
 
     // key-block range of this workgroup
     // Sequence lengths that are not a multiple of the block sizes: the copies of K/V rows past the end return zeros
@@ -511,9 +509,9 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     // kernel-argument pointer, so that these values do not occupy scalar registers during the main loop.
     const KernargPtr pe = kernarg_block();
     const int e_heads = pe->heads, e_seqlen = pe->seqlen;
-    const int eb = head / e_heads, eh = head % e_heads;
+    const int eb = fast_div(head, pe->d_heads), eh = head - eb * e_heads;
     const float l_tot = half_pair_sum(l_run);          // in units of 1/127 when PROUND == 0
-    const float vs = VBLK ? 1.f : load_scale(pe->v_scale, eb * pe->vs_sb + (eh / pe->kv_group) * pe->vs_sh, pe->scale_dtype);
+    const float vs = VBLK ? 1.f : load_scale(pe->v_scale, eb * pe->vs_sb + fast_div(eh, pe->d_kv_group) * pe->vs_sh, pe->scale_dtype);
     // (no visible key at all - an empty cache entry, or a causal row above the first key when there are fewer keys than
     // queries - gives zeros and lse = -inf; such a row's accumulators hold NaN from exp2(-inf - -inf), hence the selects)
     const bool any_key = nb_begin < nb_end && m_run > -INFINITY;

@@ -48,20 +48,18 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
     const int n_mblk = (p.seqlen + kBlockM - 1) / kBlockM;
     const int n_split = SPLIT ? p.num_splits : 1;
     const bool pair = CAUSAL && !SPLIT && p.pair_mblocks != 0;
-    const int per_head = pair ? n_mblk / 2 : n_mblk * n_split;
-    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x, per_head);
-    const int rem = wg.rem, head = wg.head;
-    const int kv_group = p.kv_group;
-    const int mb_idx = rem / n_split;
-    const int split = rem % n_split;
+    const WorkgroupJob wg = deal_workgroup(p, blockIdx.x);
+    const int rem = wg.rem, head = wg.b * p.heads + wg.h;
+    const int mb_idx = fast_div(rem, p.d_n_split);
+    const int split = rem - mb_idx * n_split;
     const int njobs = pair ? 2 : 1;
 #pragma clang loop unroll(disable)
     for (int job = 0; job < njobs; ++job) {
     if (job) __syncthreads();                    // every wave is done with the LDS of the first query block
     int mb = mb_idx;
     if (CAUSAL) mb = (pair && job) ? mb_idx : n_mblk - 1 - mb_idx;     // heaviest query blocks first
-    const int b = head / p.heads, h = head % p.heads;
-    const int hk = h / kv_group;
+    const int b = wg.b, h = wg.h;
+    const int hk = wg.hk;
 
     const int seqlen_k = keys_of_batch(p, b);
     // causal mask aligned to the bottom right corner: query row i sees keys 0 .. i + causal_off
@@ -339,14 +337,14 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
     // ---- epilogue
     const KernargPtr pe = kernarg_block();
     const int e_heads = pe->heads, e_seqlen = pe->seqlen;
-    const int eb = head / e_heads, eh = head % e_heads;
+    const int eb = fast_div(head, pe->d_heads), eh = head - eb * e_heads;
     // row sum: this wave's keys plus the partner's (the last block's barriers lie between the last use of the exchange
     // slots and this one)
     float l_tot = half_pair_sum(l_run);          // in units of 1/127 when PROUND == 0
     *(float*)(smem + xm_wr) = l_tot;
     __syncthreads();
     l_tot += *(const float*)(smem + xm_rd);
-    const float vs = VBLK ? 1.f : load_scale(pe->v_scale, eb * pe->vs_sb + (eh / pe->kv_group) * pe->vs_sh, pe->scale_dtype);
+    const float vs = VBLK ? 1.f : load_scale(pe->v_scale, eb * pe->vs_sb + fast_div(eh, pe->d_kv_group) * pe->vs_sh, pe->scale_dtype);
     // (a row without a visible key gives zeros and lse = -inf; its accumulators hold NaN from exp2(-inf - -inf), hence
     // the selects)
     const bool any_key = nb_begin < nb_end && m_run > -INFINITY;

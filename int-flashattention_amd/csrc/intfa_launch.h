@@ -16,12 +16,35 @@ struct LaunchSel {
     bool dump_s;     // full-int8 only: export int32 S and stop
 };
 
+inline FastDiv make_fast_div(int d) {
+    int l = 0;
+    while ((1ll << l) < (long long)d) ++l;                   // ceil(log2 d), d >= 1
+    const unsigned s = 31u + (unsigned)l;
+    const unsigned long long m = ((1ull << s) + (unsigned long long)d - 1) / (unsigned long long)d;   // < 2^32
+    return {(uint32_t)m, (uint32_t)s};
+}
+// Fills the workgroup -> work mapping of a launch of `grid` workgroups (grid = batch * heads * workgroups per head).
+inline KParams finish_mapping(const KParams& kp, int grid) {
+    KParams k = kp;
+    const int n_split = kp.num_splits > 1 ? kp.num_splits : 1;
+    k.per_head = grid / (kp.batch * kp.heads);
+    k.heads_kv = kp.heads / kp.kv_group;
+    k.xcd_deal = ((kp.batch * k.heads_kv) & 7) == 0 ? 1 : 0;
+    k.d_per_kv = make_fast_div(k.per_head * kp.kv_group);
+    k.d_heads_kv = make_fast_div(k.heads_kv);
+    k.d_per_head = make_fast_div(k.per_head);
+    k.d_n_split = make_fast_div(n_split);
+    k.d_heads = make_fast_div(kp.heads);
+    k.d_kv_group = make_fast_div(kp.kv_group);
+    return k;
+}
+
 // One workgroup per (batch, head, 128-row query block, split); causal single-pass launches pair the query blocks.
 // `column_halves`: workgroups per query block (2 where a kernel splits the output columns over two workgroups).
 template <typename K> inline int launch_kernel(K kernel, const KParams& kp, hipStream_t stream, int threads = kThreads,
                                                int column_halves = 1) {
     const int grid = kp.batch * kp.heads * ((kp.seqlen + kBlockM - 1) / kBlockM) * kp.num_splits / (kp.pair_mblocks ? 2 : 1) * column_halves;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), 0, stream, kp);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), 0, stream, finish_mapping(kp, grid));
     return (int)hipGetLastError();
 }
 
