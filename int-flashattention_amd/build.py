@@ -7,6 +7,9 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+if HERE not in sys.path:
+    sys.path.insert(0, HERE)
+import spill_check  # noqa: E402  (a sibling module; this file also runs as a script)
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libintfa.so")
 # -packed-fp32-ops is switched off on purpose: the compiler must not form v_pk_*_f32 from the float code.
@@ -43,15 +46,30 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
     objs = [os.path.join(objdir, os.path.basename(s)[:-4] + ".o") for s in srcs]
 
     def compile_one(pair):
+        # -save-temps=obj leaves the device assembly beside the object: it is scanned for register spills that lose lanes
+        # (spill_check.py) and removed again with the other intermediate files
         src, obj = pair
-        cmd = ["hipcc", *FLAGS, "-c", src, "-o", obj]
+        cmd = ["hipcc", *FLAGS, "-save-temps=obj", "-c", src, "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed for {src}:\n{r.stderr[-4000:]}")
-        return obj
+        stem = os.path.basename(src)[:-4]
+        findings = []
+        for f in os.listdir(objdir):
+            if not f.startswith(stem + "-") and not f.startswith(stem + ".hip-"):
+                continue
+            path = os.path.join(objdir, f)
+            if f.endswith("gfx950.s"):
+                with open(path) as fh:
+                    findings = [f"{os.path.basename(src)}: {x}" for x in spill_check.scan(fh.read())]
+            os.remove(path)
+        return findings
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        list(ex.map(compile_one, zip(srcs, objs)))
+        findings = [x for fs in ex.map(compile_one, zip(srcs, objs)) for x in fs]
+    if findings:
+        raise RuntimeError("the compiler placed register spills where lanes are masked off (wrong results for those lanes):\n  "
+                           + "\n  ".join(findings[:20]))
     r = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", OUT], capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")

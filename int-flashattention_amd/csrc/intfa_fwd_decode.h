@@ -111,7 +111,9 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
     auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
     // VBLK: fp32 channel scales of a key block; thread 128 + c fetches channel c
     const int vs_c = tid - 128;
-    const bool vs_thread = VBLK && vs_c >= 0 && vs_c < D;
+    // (per-wave tests, scalar branches: see fwd_full_int8_kernel)
+    const bool ks_wave = wave < BN / 64;
+    const bool vs_thread = VBLK && wave >= 2 && (wave - 2) * 64 < D;
     const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + (vs_thread ? vs_c : 0));
     auto load_vs = [&](int nb) __attribute__((always_inline)) -> float {
         if (!VBLK) return 0.f;
@@ -160,7 +162,7 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
         float vs_next = 0.f;
         if (more) {
             issue_loads(nb + NBS, BUF ^ 1);
-            if (tid < BN) ks_next = load_ks(nb + NBS);
+            if (ks_wave) ks_next = load_ks(nb + NBS);
             if (vs_thread) vs_next = load_vs(nb + NBS);
         }
         // -------- S^T of this wave's 32 keys, dequantise, partial row maximum
@@ -274,13 +276,13 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
         }
         if (NBS == 1) l_run = fmaf(l_run, alpha, lsum);
         else l_run = blk_a ? fmaf(l_run, alpha, lsum) * alpha_b : fmaf(l_run * alpha, alpha_b, lsum);
-        if (more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
+        if (more && ks_wave) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
         if (more && vs_thread) *(float*)(smem + vs_wr + (BUF ^ 1) * D * 4) = vs_next;
     };
 
     if (nb_begin < nb_end) {
         issue_loads(nb_begin, 0);
-        if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(load_ks(nb_begin));
+        if (ks_wave) *(float*)(smem + ks_wr) = cvt_ks(load_ks(nb_begin));
         if (vs_thread) *(float*)(smem + vs_wr) = load_vs(nb_begin);
         int nb = nb_begin;
         while (true) {

@@ -113,8 +113,9 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
     };
     // k_scale of a step: thread t < 128 fetches the scale of key t; converted to fp32 when stored to LDS
     const KScaleSource ks_src(p, b, hk, seqlen_k);
+    const bool ks_wave = wave < BN / 64;              // threads 0 .. BN-1 fetch one k_scale each (a scalar test: see fwd_full_int8_kernel)
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
-        return (!QK_INT8 || tid >= BN) ? 0u : ks_src.load(nb * BNB + tid);
+        return (!QK_INT8 || !ks_wave) ? 0u : ks_src.load(nb * BNB + tid);
     };
     auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
 
@@ -263,14 +264,14 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
         }
         if (NBS == 1) l_run = fmaf(l_run, alpha_a, lsum);
         else l_run = blk_a ? fmaf(l_run, alpha_a, lsum) * alpha_b : fmaf(l_run * alpha_a, alpha_b, lsum);
-        if (QK_INT8 && more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
+        if (QK_INT8 && more && ks_wave) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
     };
 
     if (nb_begin < nb_end) {
         issue_loads(nb_begin, 0);
         if (QK_INT8) {
             const uint32_t s0 = load_ks(nb_begin);
-            if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
+            if (ks_wave) *(float*)(smem + ks_wr) = cvt_ks(s0);
         }
         int nb = nb_begin;
         while (true) {

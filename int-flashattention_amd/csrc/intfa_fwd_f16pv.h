@@ -122,8 +122,9 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
         issue_tile_load<VROW, SWZ_V16, BN>(v_rsrc, (uint32_t)(nb * BN) * v_sn, v_sn, lds0 + OFF_V + buf * VT, wave, v_lane);
     };
     const KScaleSource ks_src(p, b, hk, seqlen_k);
+    const bool ks_wave = wave == 0;                  // threads 0 .. 63 fetch one k_scale each (a scalar test: see fwd_full_int8_kernel)
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t {
-        return (!QK_INT8 || tid >= BN) ? 0u : ks_src.load(nb * BN + tid);
+        return (!QK_INT8 || !ks_wave) ? 0u : ks_src.load(nb * BN + tid);
     };
     auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
 
@@ -289,14 +290,14 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
         uint32_t ks_next = 0;
         if (more) { issue_loads(nb + 1, BUF ^ 1); ks_next = load_ks(nb + 1); }
         compute(buf_tag, diag_tag, nb, gw, lim, lim_lo);
-        if (QK_INT8 && more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
+        if (QK_INT8 && more && ks_wave) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
     };
 
     if (nb_begin < nb_end) {
         issue_loads(nb_begin, 0);
         if (QK_INT8) {
             const uint32_t s0 = load_ks(nb_begin);
-            if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
+            if (ks_wave) *(float*)(smem + ks_wr) = cvt_ks(s0);
         }
         const int diag_first = (mb * kBlockM + causal_off + 1) / BN;   // first block with a key hidden from the block's first row
         const int diag_begin = diag_first < 0 ? 0 : diag_first;

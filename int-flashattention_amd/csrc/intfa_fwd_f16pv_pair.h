@@ -236,7 +236,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_f16pv_pair_kernel(const K
         for (int u = 0; u < 2; ++u) { vfo[1][u] = load_vfrag(v_own, 1, u); vfp[1][u] = load_vfrag(v_oth, 1, u); }
         if (hf == 0) {                           // the next block's K tile and k_scale
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            if (QK_INT8 && more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = ks_src.cvt(ks_next);
+            if (QK_INT8 && more && wave == 0) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = ks_src.cvt(ks_next);
         }
         __syncthreads();                         // ---- B3
         pfp[0] = *(const v4i*)(smem + xp_rd);
@@ -286,7 +286,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_f16pv_pair_kernel(const K
         if (hf == 0) issue_k(nb_begin, 0); else issue_v(nb_begin, 0);
         if (QK_INT8) {
             const uint32_t s0 = load_ks(nb_begin);
-            if (tid < BN) *(float*)(smem + ks_wr) = ks_src.cvt(s0);
+            if (wave == 0) *(float*)(smem + ks_wr) = ks_src.cvt(s0);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();

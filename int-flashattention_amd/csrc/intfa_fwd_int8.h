@@ -146,8 +146,13 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
     auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
     // VBLK: channel scales of a key block; thread 128 + c fetches the scale of this workgroup's channel c.  A scale
     // row covers vs_g key blocks.
+    // (Which threads fetch scales is decided per WAVE, from the wave index held in a scalar register: the branches
+    // below are scalar branches that leave the exec mask alone.  A per-thread test of threadIdx would mask lanes off, and
+    // a register spill or reload that the compiler places in the block where such lanes rejoin runs before the mask is
+    // restored there: the lanes that were off lose the value.)
+    const bool ks_wave = wave < BN / 64;             // threads 0 .. BN-1: one k_scale each
     const int vs_c = tid - 128;
-    const bool vs_thread = VBLK && vs_c >= 0 && vs_c < DV;
+    const bool vs_thread = VBLK && wave >= 2 && (wave - 2) * 64 < DV;   // threads 128 .. 128 + DV - 1: one channel each
     // (these scales are fp32 whatever the type of the per-token scales, as in the reference's kernel)
     const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + (vs_thread ? vs_c : 0));
     // (VBLK == 2: scale rows 2 nb and 2 nb + 1; the second one does not exist when the sequence ends inside the block's
@@ -456,7 +461,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
             }
         }
         compute(buf_tag, diag_tag, nb, more, gw, lim, lim_lo);
-        if (more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
+        if (more && ks_wave) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
         if (more && vs_thread) {
 #pragma unroll
             for (int sub = 0; sub < VSUB; ++sub) *(float*)(smem + vs_wr + ((BUF ^ 1) * VSUB + sub) * DV * 4) = vs_next[sub];
@@ -469,7 +474,7 @@ __global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParam
         issue_loads(nb_begin, 0);
         {
             const uint32_t s0 = load_ks(nb_begin);
-            if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
+            if (ks_wave) *(float*)(smem + ks_wr) = cvt_ks(s0);
             if (vs_thread) {
 #pragma unroll
                 for (int sub = 0; sub < VSUB; ++sub) *(float*)(smem + vs_wr + sub * DV * 4) = load_vs(nb_begin, sub);

@@ -104,8 +104,13 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t { return ks_src.load(nb * BN + ks_key); };   // raw bits
     auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
     // VBLK: thread 256 + c fetches the fp32 scale of channel c of the key block's scale row (vs_g key blocks per row)
+    // (Which threads fetch scales is decided per WAVE, from the wave index held in a scalar register: the branches
+    // below are scalar branches that leave the exec mask alone.  A per-thread test of threadIdx would mask lanes off, and
+    // a register spill or reload that the compiler places in the block where such lanes rejoin runs before the mask is
+    // restored there: the lanes that were off lose the value.)
+    const bool ks_wave = wave == 0;              // threads 0 .. 63: one k_scale each
     const int vs_c = tid - 256;
-    const bool vs_thread = VBLK && vs_c >= 0;
+    const bool vs_thread = VBLK && hf == 1;      // threads 256 .. 511: one channel each
     const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + (vs_thread ? vs_c : 0));
     auto load_vs = [&](int nb) __attribute__((always_inline)) -> float {
         if (!VBLK) return 0.f;
@@ -252,7 +257,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
         vfp[1] = load_vfrag(v_oth, 1);
         if (hf == 0) {                           // the next block's K tile and k_scale
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            if (more && tid < BN) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
+            if (more && ks_wave) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
         }
         __syncthreads();                         // ---- B3
         const v4i p8p = *(const v4i*)(smem + xp_rd);
@@ -313,7 +318,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
         issue_loads(nb_begin, 0);
         {
             const uint32_t s0 = load_ks(nb_begin);
-            if (tid < BN) *(float*)(smem + ks_wr) = cvt_ks(s0);
+            if (ks_wave) *(float*)(smem + ks_wr) = cvt_ks(s0);
             if (vs_thread) vs_pend = load_vs(nb_begin);
         }
         if (hf == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -53,6 +53,8 @@ def test_quant_perblock_channel_strided_input():
     (1, 2, 512, 128, True, 2),         # one scale row per two key blocks of the kernel
     (1, 2, 256, 256, False, 1),        # head_dim 256: 64-key blocks, column halves
     (1, 2, 320, 256, True, 2),
+    (1, 2, 384, 256, True, 1),         # three query blocks: one per workgroup, heaviest first
+    (2, 3, 512, 256, True, 1),         # four query blocks: paired in one workgroup
     (1, 3, 300, 128, False, 1),        # ragged length: the last scale row covers 44 keys
     (1, 2, 97, 64, True, 1),
     # 64-key scale rows under the 128-key block: the granularity of the reference's CUDA kernel (kBlockN = 64 at
@@ -70,13 +72,15 @@ def test_blocked_v_scale_matches_oracle(B, H, N, D, causal, mult, p_round):
     vsb = int(bn * mult)
     x = blocked_inputs(B, H, N, D, 80, vsb)
     sm = D ** -0.5
-    o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), causal, sm, p_round=p_round,
-                              v_scale_block=vsb)
+    o, lse = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), causal, sm, p_round=p_round,
+                                   v_scale_block=vsb, return_lse=True)
     torch.cuda.synchronize()
     assert o.dtype == torch.float16 and o.shape == (B, H, N, D)
-    ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=bn,
-                                v_scale_block=vsb)
+    ref, lse_ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=bn,
+                                         v_scale_block=vsb, return_lse=True)
     assert max_abs(o, ref) <= MAX_ABS and mean_rel(o, ref) <= MEAN_REL
+    # every row's LSE (it does not depend on V or its scales; a row that lands in another row's slot shows here only)
+    assert (lse.cpu() - lse_ref).abs().max().item() <= 1e-3
     same = ref if p_round == "reference" else O.attention_full_int8(
         x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=bn, v_scale_block=vsb,
         p_requant=O.p_requant_rne)
