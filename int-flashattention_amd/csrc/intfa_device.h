@@ -335,6 +335,10 @@ __device__ __forceinline__ void out_stage_flush(const char* stage, char* g_row0,
     }
 }
 
+// fp32 -> bf16 in hardware (v_cvt_pk_bf16_f32 converts two values per instruction, round-to-nearest-even): what the
+// attention kernels use for P and for the output.  (The quantisers keep the integer form below: they reproduce another
+// library's results bit for bit, NaN patterns included.)
+__device__ __forceinline__ short f32_to_bf16(float f) { return __builtin_bit_cast(short, (__bf16)f); }
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {   // round-to-nearest-even
     uint32_t u = __builtin_bit_cast(uint32_t, f);
     u += 0x7fffu + ((u >> 16) & 1u);

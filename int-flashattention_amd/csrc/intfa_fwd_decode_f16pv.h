@@ -329,7 +329,7 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
                 } else {
                     v4s o;
 #pragma unroll
-                    for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(seen ? o_acc[j][4 * a4 + b4] * inv : 0.f);
+                    for (int b4 = 0; b4 < 4; ++b4) o[b4] = f32_to_bf16(seen ? o_acc[j][4 * a4 + b4] * inv : 0.f);
                     *(v4s*)(orow + d0 * 2) = o;
                 }
             }

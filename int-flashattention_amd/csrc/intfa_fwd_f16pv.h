@@ -23,7 +23,7 @@ __device__ __forceinline__ v8h pack_p_f16(const float* e) {
 __device__ __forceinline__ v8bf pack_p_bf16(const float* e) {
     v8bf r;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) r[i] = __builtin_bit_cast(__bf16, (uint16_t)f32_to_bf16_bits(e[i]));
+    for (int i = 0; i < 8; ++i) r[i] = (__bf16)e[i];
     return r;
 }
 
@@ -375,7 +375,7 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
             } else {
                 v4s o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(any_key ? o_acc[dt][4 * a4 + b4] * inv : 0.f);
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = f32_to_bf16(any_key ? o_acc[dt][4 * a4 + b4] * inv : 0.f);
                 out_stage_put<DV>(stage, lq_e, d0, __builtin_bit_cast(v2i, o));
             }
         }

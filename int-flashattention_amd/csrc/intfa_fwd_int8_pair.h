@@ -396,7 +396,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) fwd_full_int8_pair_kernel(con
             } else {
                 v4s o;
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4) o[b4] = (short)f32_to_bf16_bits(any_key ? o_acc[dt][4 * a4 + b4] * out_scale : 0.f);
+                for (int b4 = 0; b4 < 4; ++b4) o[b4] = f32_to_bf16(any_key ? o_acc[dt][4 * a4 + b4] * out_scale : 0.f);
                 out_stage_put<DVW>(stage, lq_e, d0, __builtin_bit_cast(v2i, o));
             }
         }

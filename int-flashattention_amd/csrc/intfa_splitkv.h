@@ -54,7 +54,7 @@ __global__ void __launch_bounds__(256) splitkv_combine_kernel(const KParams p) {
     } else {
         v4s o;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = (short)f32_to_bf16_bits(acc[i]);
+        for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16(acc[i]);
         *(v4s*)orow = o;
     }
     if (p.lse != nullptr && sub == 0) p.lse[row] = lse;
