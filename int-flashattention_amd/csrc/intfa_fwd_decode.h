@@ -276,6 +276,9 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
         }
         if (NBS == 1) l_run = fmaf(l_run, alpha, lsum);
         else l_run = blk_a ? fmaf(l_run, alpha, lsum) * alpha_b : fmaf(l_run * alpha, alpha_b, lsum);
+        // (the raw scale is made opaque here, behind the step's last barrier: its conversion waits for the load, and with it
+        // for the next step's tile copies that were issued ahead of it - that wait belongs at the end of the step)
+        asm volatile("" : "+v"(ks_next));
         if (more && ks_wave) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
         if (more && vs_thread) *(float*)(smem + vs_wr + (BUF ^ 1) * D * 4) = vs_next;
     };

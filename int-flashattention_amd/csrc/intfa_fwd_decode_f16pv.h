@@ -264,6 +264,9 @@ __global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_ke
         }
         if (NBS == 1) l_run = fmaf(l_run, alpha_a, lsum);
         else l_run = blk_a ? fmaf(l_run, alpha_a, lsum) * alpha_b : fmaf(l_run * alpha_a, alpha_b, lsum);
+        // (the raw scale is made opaque here, behind the step's last barrier: its conversion waits for the load, and with it
+        // for the next step's tile copies that were issued ahead of it - that wait belongs at the end of the step)
+        if (QK_INT8) asm volatile("" : "+v"(ks_next));
         if (QK_INT8 && more && ks_wave) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
     };
 
