@@ -84,6 +84,7 @@ def test_qk_int32_extreme_values():
     (1, 2, 1024, 128, False),
     (1, 2, 256, 256, False),       # head_dim 256 runs with 64-key blocks
     (2, 2, 384, 256, True),
+    (1, 2, 512, 256, True),        # four query blocks: two per workgroup
 ])
 @pytest.mark.parametrize("p_round", ["rne", "reference"])
 def test_full_int8_matches_oracle(B, H, N, D, causal, p_round):
@@ -91,10 +92,12 @@ def test_full_int8_matches_oracle(B, H, N, D, causal, p_round):
     sm = D ** -0.5
     bn = M.block_n("full", D)
     assert bn == (128 if D <= 128 else 64)
-    o = run_full(x, causal, sm, p_round=p_round)
+    o, lse = run_full(x, causal, sm, p_round=p_round, return_lse=True)
     assert o.dtype == torch.float16 and o.shape == (B, H, N, D) and o.is_contiguous()
-    ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=bn)
+    ref, lse_ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=bn,
+                                         return_lse=True)
     assert max_abs(o, ref) <= MAX_ABS and mean_rel(o, ref) <= MEAN_REL
+    assert (lse.cpu() - lse_ref).abs().max().item() <= 1e-3         # every row's LSE in its own slot
     same = ref if p_round == "reference" else O.attention_full_int8(
         x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=bn, p_requant=O.p_requant_rne)
     assert_same_rounding(o, same)
@@ -230,12 +233,14 @@ def test_half_int8_matches_oracle(B, H, N, D, causal, dtype):
     x = quantised(B, H, N, D, seed=31, dtype=dtype)
     sm = D ** -0.5
     bn = M.block_n("half", D)
-    o = M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), causal, sm)
+    o, lse = M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), causal, sm, return_lse=True)
     torch.cuda.synchronize()
     assert o.dtype == dtype and o.shape == (B, H, N, D)
-    ref = O.attention_int8(x["q8"], x["k8"], x["v"], x["qs"], x["ks"], causal, sm, block_n=bn, out_dtype=dtype)
+    ref, lse_ref = O.attention_int8(x["q8"], x["k8"], x["v"], x["qs"], x["ks"], causal, sm, block_n=bn, out_dtype=dtype,
+                                    return_lse=True)
     ma, mr = _ulp_bounds(dtype)
     assert max_abs(o, ref) <= ma and mean_rel(o, ref) <= mr
+    assert (lse.cpu() - lse_ref).abs().max().item() <= 2e-3
     if dtype == torch.float16:
         exact = O.attention_exact(x["q"], x["k"], x["v"], causal, sm)
         assert max_abs(o, exact) <= 4e-2 and mean_rel(o, exact) <= 2e-2     # int8 Q/K quantisation error itself
@@ -246,12 +251,13 @@ def test_fp16_attention_matches_oracle(B, H, N, D, causal, dtype):
     q, k, v, _ = O.make_inputs(B, H, N, D, seed=32, dtype=dtype)
     sm = D ** -0.5
     bn = M.block_n("fp", D)
-    o = M.attention(*gpu(q, k, v), causal, sm)
+    o, lse = M.attention(*gpu(q, k, v), causal, sm, return_lse=True)
     torch.cuda.synchronize()
     assert o.dtype == dtype and o.shape == (B, H, N, D)
-    ref = O.attention_fp(q, k, v, causal, sm, block_n=bn)
+    ref, lse_ref = O.attention_fp(q, k, v, causal, sm, block_n=bn, return_lse=True)
     ma, mr = _ulp_bounds(dtype)
     assert max_abs(o, ref) <= ma and mean_rel(o, ref) <= mr
+    assert (lse.cpu() - lse_ref).abs().max().item() <= 2e-3
     exact = O.attention_exact(q, k, v, causal, sm)
     assert max_abs(o, exact) <= (2e-3 if dtype == torch.float16 else 1.6e-2)
 
