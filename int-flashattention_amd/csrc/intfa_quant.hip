@@ -9,6 +9,7 @@
 // owns 8 consecutive elements (one 16-byte load, one 8-byte store) and d / 8 lanes share a row.
 #include "../../include/intfa.h"
 #include "intfa_device.h"
+#include "intfa_launch.h"
 
 using namespace intfa;
 
@@ -86,6 +87,7 @@ struct QuantParams {
     int64_t sb, sh, sn;             // bytes
     int32_t heads, seqlen, head_dim;
     int64_t rows;                   // batch * heads * seqlen
+    FastDiv d_seqlen, d_heads;      // row index -> (batch, head, position) without a run-time division per row
 };
 
 // ---- per token: LPR = d / 8 lanes per row, reduction of the row maximum inside those lanes
@@ -94,8 +96,8 @@ constexpr int kRowsInFlight = 8;    // independent 16-byte loads a lane has in f
 // rows are numbered (batch, head, position) in that order; the count fits 31 bits (checked on the host), so the index
 // arithmetic is 32-bit
 __device__ __forceinline__ const char* row_ptr(const QuantParams& p, uint32_t row, int sub, uint32_t* bh_out) {
-    const uint32_t bh = row / (uint32_t)p.seqlen, n = row - bh * (uint32_t)p.seqlen;
-    const uint32_t b = bh / (uint32_t)p.heads, h = bh - b * (uint32_t)p.heads;
+    const uint32_t bh = (uint32_t)fast_div((int)row, p.d_seqlen), n = row - bh * (uint32_t)p.seqlen;
+    const uint32_t b = (uint32_t)fast_div((int)bh, p.d_heads), h = bh - b * (uint32_t)p.heads;
     *bh_out = bh;
     return p.x + b * p.sb + h * p.sh + n * p.sn + sub * 16;
 }
@@ -284,6 +286,8 @@ int check(const void* x, const void* q8, const void* scale, int64_t sb, int64_t 
     qp->heads = heads; qp->seqlen = seqlen; qp->head_dim = head_dim;
     qp->rows = (int64_t)batch * heads * seqlen;
     if (qp->rows >= (1ll << 31) - (1 << 24)) return INTFA_ERR_SHAPE;      // 32-bit row indices, with room for the strides
+    qp->d_seqlen = make_fast_div(seqlen);
+    qp->d_heads = make_fast_div(heads);
     return INTFA_OK;
 }
 
@@ -306,6 +310,7 @@ struct AppendParams {
     const int32_t* seqlens_k;
     int32_t seqlen_filled, heads, seqlen_new, seqlen_cache, head_dim;
     int64_t rows;                                 // batch * heads * seqlen_new
+    FastDiv d_seqlen_new, d_heads;
 };
 
 template <int DT, int LPR, bool IS_V> __global__ void __launch_bounds__(256) kv_append_kernel(const AppendParams p) {
@@ -321,9 +326,9 @@ template <int DT, int LPR, bool IS_V> __global__ void __launch_bounds__(256) kv_
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint32_t row = row0 + u * step;
-            const uint32_t bh = row / (uint32_t)p.seqlen_new;
+            const uint32_t bh = (uint32_t)fast_div((int)row, p.d_seqlen_new);
             iq[u] = row - bh * (uint32_t)p.seqlen_new;
-            bq[u] = bh / (uint32_t)p.heads; hq[u] = bh - bq[u] * (uint32_t)p.heads;
+            bq[u] = (uint32_t)fast_div((int)bh, p.d_heads); hq[u] = bh - bq[u] * (uint32_t)p.heads;
             raw[u] = row < rows ? *(const v4i*)(s.x + bq[u] * s.xb + hq[u] * s.xh + iq[u] * s.xn + sub * 16) : (v4i){0, 0, 0, 0};
         }
 #pragma unroll
@@ -482,6 +487,8 @@ int intfa_kvcache_append_int8(const intfa_append_params* a, void* stream) {
     ap.seqlens_k = a->seqlens_k;
     ap.seqlen_filled = a->seqlen_filled;
     ap.heads = a->heads_kv; ap.seqlen_new = a->seqlen_new; ap.seqlen_cache = a->seqlen_cache; ap.head_dim = d;
+    ap.d_seqlen_new = make_fast_div(a->seqlen_new);
+    ap.d_heads = make_fast_div(a->heads_kv);
     ap.rows = rows;
     hipStream_t st = (hipStream_t)stream;
 #define INTFA_CALL(LPR) do { const int g = grid_for(rows, 256 / LPR); \
