@@ -54,7 +54,7 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed for {src}:\n{r.stderr[-4000:]}")
         stem = os.path.basename(src)[:-4]
-        findings = []
+        findings, scanned = [], False
         for f in os.listdir(objdir):
             if not f.startswith(stem + "-") and not f.startswith(stem + ".hip-"):
                 continue
@@ -62,7 +62,10 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
             if f.endswith("gfx950.s"):
                 with open(path) as fh:
                     findings = [f"{os.path.basename(src)}: {x}" for x in spill_check.scan(fh.read())]
+                scanned = True
             os.remove(path)
+        if not scanned:      # (a compiler that names its intermediate files otherwise must not pass unchecked)
+            raise RuntimeError(f"no device assembly found for {src}: the spill scan did not run")
         return findings
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
