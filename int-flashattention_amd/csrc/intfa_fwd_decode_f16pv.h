@@ -2,21 +2,24 @@
 //
 // Same arithmetic as fwd_f16pv_kernel (flash_atten_int8.py:9-66, flash_atten_fp.py:9-60 per 64-key block: S, running
 // max, P = exp2(S c - m) cast to V's 16-bit type, fp32 accumulator scaled by alpha and P V added on top), other division
-// of labour - the one of fwd_decode_full_int8_kernel.  One workgroup owns 32 query rows; its four waves share the keys:
-// a step covers TWO consecutive 64-key blocks A and B (128 keys),
+// of labour - the one of fwd_decode_full_int8_kernel.  One workgroup owns 32 query rows; its four waves share the keys.
+//
+// Head_dim 64: a step covers TWO consecutive 64-key blocks A and B (128 keys),
 //   * wave w computes S^T for keys 32w .. 32w+31 of the step (waves 0, 1: block A; waves 2, 3: block B), dequantises and
 //     takes the partial row maxima;
 //   * the four partial maxima meet in LDS (barrier); every wave then knows both blocks' running maxima
 //     m_A = max(m, max_A), m_B = max(m_A, max_B) and both factors alpha_A = 2^(m - m_A), alpha_B = 2^(m_A - m_B);
 //   * wave w exponentiates its 32 keys against its block's maximum, casts to 16 bits and publishes two MFMA operands
 //     in LDS (barrier);
-//   * wave w owns 32 output columns: O = (O alpha_A + P_A V_A) alpha_B + P_B V_B with all eight operands.
+//   * waves 0 and 1 own 32 output columns each: O = (O alpha_A + P_A V_A) alpha_B + P_B V_B with all eight operands.
+// Head_dim 128 and 256: a step is ONE 64-key block.  Waves 0 and 1 compute S^T and P for its two 32-key sub-tiles,
+// waves 2 and 3 only pass the barriers in that phase (the pass is bound by the stream of K and V, not by the arithmetic),
+// every wave owns one (two at head_dim 256) 32-column output tile.  The smaller step is what the stream wants there: 24
+// to 32 KiB of tiles per step let two or three workgroups share a compute unit at head_dim 128 (6.0 TB/s of K+V against
+// 5.4 - 5.9 with 128-key steps and one workgroup), and at head_dim 256 two steps of 128 keys would not fit the LDS.
 // Every block is evaluated with the same maximum, the same P and the same order of MFMA steps as in the general kernel;
 // only the row sums are added in another order (per wave, joined in the epilogue).  K/V tiles of a step are
 // double-buffered in LDS and the whole next step is requested at the start of a step.
-// Head_dim 256: 128 keys of 16-bit V (and K) do not fit the LDS twice, so a step is ONE 64-key block there: waves 0 and 1
-// compute S^T and P for its two 32-key sub-tiles, waves 2 and 3 only wait at the barriers in that phase (the pass is
-// bound by the stream of K and V, not by the arithmetic), and every wave owns two 32-column output tiles.
 #pragma once
 #include "intfa_device.h"
 #include "intfa_launch.h"
@@ -27,11 +30,11 @@ namespace intfa {
 // QK_INT8: int8 Q/K with per-token scales (half-int8) or 16-bit Q/K.  IO_DT: type of V, P and the output (and of Q/K
 // when !QK_INT8): 0 fp16, 1 bf16.  The causal mask is a run-time switch here (p.causal).
 template <bool QK_INT8, int D, int IO_DT, bool SPLIT>
-__global__ void __launch_bounds__(kThreads, D == 64 ? 2 : 1) fwd_decode_f16pv_kernel(const KParams p) {
+__global__ void __launch_bounds__(kThreads, D == 256 ? 1 : (D == 128 && QK_INT8) ? 3 : 2) fwd_decode_f16pv_kernel(const KParams p) {
     static_assert(D == 64 || D == 128 || D == 256, "head dims 64, 128 and 256");
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int BNB = kBlockN16;                    // key block of the arithmetic
-    constexpr int NBS = D <= 128 ? 2 : 1;             // key blocks per step
+    constexpr int NBS = D <= 64 ? 2 : 1;              // key blocks per step
     constexpr int BN = NBS * BNB;                     // keys per step
     constexpr int QKW = BN / 32;                      // waves with a 32-key sub-tile of S^T (all four, or waves 0 and 1)
     constexpr int NG = BN / 16;                       // 16-key MFMA steps of P V per step (two per wave's sub-tile)
