@@ -265,8 +265,8 @@ int intfa_fwd_suggest_splits(const intfa_fwd_params* p, int variant, int num_cus
     int64_t wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kBlockM - 1) / kBlockM);
     if (decode_shaped(variant, p->seqlen, p->head_dim, variant == INTFA_VARIANT_FULL_INT8 && p->v_scale_block > 0)) {
         wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kDecodeRows - 1) / kDecodeRows);
-        // 128 KiB of tiles and more: one workgroup per compute unit
-        if ((variant != INTFA_VARIANT_FULL_INT8 && p->head_dim == 128) || p->head_dim == 256) slots = cus;
+        // head_dim 256: 96 KiB and more of tiles, one workgroup per compute unit
+        if (p->head_dim == 256) slots = cus;
     }
     else if (p->head_dim == 256) wgs *= 2;     // full-int8: eight-wave workgroups, one per compute unit; the others: column halves
     if (wgs * 5 >= slots * 4) return 1;                                        // at least 80 % of the slots are used anyway

@@ -184,6 +184,11 @@ def test_split_count_heuristic():
     assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 0, 256) == 16             # 64 key blocks, four per split
     assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 1, 256) == 32             # 64-key blocks: 128 of them
     assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 0, 0) == 16               # default device size
+    p.batch, p.heads, p.seqlen_k = 2, 64, 4096                                      # 128 decode workgroups
+    assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 1, 256) == 4              # head_dim 128: two workgroups per CU
+    p.head_dim = 256
+    assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 1, 256) == 2              # head_dim 256: one per CU
+    p.batch, p.heads, p.head_dim = 1, 8, 128
     p.seqlen_k = 256
     assert lib.intfa_fwd_suggest_splits(ctypes.byref(p), 0, 256) == 1              # too few key blocks to split
     p.batch, p.heads, p.seqlen, p.seqlen_k = 1, 32, 1024, 0
