@@ -360,6 +360,14 @@ __device__ __forceinline__ float half_pair_sum(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// v for a visible key, -inf for a hidden one (key index k_r past the lane's last visible index `last`), without a
+// compare and select: min with a threshold that is +inf or -inf by the sign of last - k_r.  No condition registers,
+// so the statement cannot be merged with a wave-uniform test around it into a select per element.
+__device__ __forceinline__ float hide_past(float v, int last, int k_r) {
+    const uint32_t t = (uint32_t)(last - k_r);
+    return __builtin_fminf(v, __builtin_bit_cast(float, (t & 0x80000000u) | 0x7f800000u));
+}
+
 // The reference's requantisation of P (flash_atten_full_int8.py:49-51) for the 16 probabilities a lane holds of one 32-key
 // sub-tile, in the reference's own fp16 operations: fp16(p) (round to nearest even) * 127 -> fp16, + 0.5 -> fp16,
 // truncating conversion to an integer.  The multiply and the add are the packed fp16 instructions (two values each; kept

@@ -146,7 +146,7 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
     const uint32_t xp_rd = OFF_XP + 16 * lane;                       // + 1024 per wave
     const uint32_t vs_wr = OFF_VS + 4 * (vs_thread ? vs_c : 0);
     const uint32_t vs_rd = OFF_VS + 16 * lh;                         // + 4 * (32*dt + 8*a4) per read
-    const bool own_tile0 = wave < DT;                                // head_dim 64: waves 2 and 3 own no output tile
+    const bool own_tile0 = DT >= 4 || wave < DT;                     // head_dim 64: waves 2 and 3 own no output tile
     // the last visible key of the first row of this query block, and of the lane's row
     const int first_lim = p.causal ? (fold ? 0 : mb * kDecodeRows) + causal_off : 0x3fffffff;
     const int row_lim = p.causal ? (fold ? q_row % fold : q_row) + causal_off : 0x3fffffff;
@@ -198,12 +198,16 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
         const int last_key = (row_lim < key_end - 1 ? row_lim : key_end - 1) - key0;
         const int key_lim = last_key + 1 - 32 * wave - 4 * lh;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            float v = (float)sacc[r] * kk[r >> 2][r & 3];
-            if (tail && 8 * (r >> 2) + (r & 3) >= key_lim) v = -INFINITY;
-            x[r] = v;
-            mx = fmaxf(mx, v);
+        for (int r = 0; r < 16; ++r) x[r] = (float)sacc[r] * kk[r >> 2][r & 3];
+        if (tail) {
+            // (a branch of its own, kept one by the empty statement: folded into the loop above, the test would put a
+            // compare and a select on every element of every step)
+            asm volatile("");
+#pragma unroll
+            for (int r = 0; r < 16; ++r) x[r] = hide_past(x[r], key_lim - 1, 8 * (r >> 2) + (r & 3));
         }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, x[r]);
         mx = half_pair_max(mx);
         if (lh == 0) *(float*)(smem + xm_wr) = mx;
         __syncthreads();                                   // the four partial maxima are in LDS

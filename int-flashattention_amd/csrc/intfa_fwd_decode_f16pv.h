@@ -132,7 +132,7 @@ __global__ void __launch_bounds__(kThreads, D == 256 ? 1 : (D == 128 && QK_INT8)
     const int g16 = lane >> 4, s16 = lane & 15;
     const int v_row0 = 4 * lh + (s16 >> 2);           // + 8 for the second load, + 16 per MFMA step
     const int v_swz = swz_v16<VROW>(v_row0) & (VCH - 1);
-    const bool own_tile = wave < DT;                  // head_dim 64: waves 2 and 3 own no output tile
+    const bool own_tile = DT >= 4 || wave < DT;       // head_dim 64: waves 2 and 3 own no output tile
     const bool qk_wave = wave < QKW;                  // this wave computes a sub-tile of S^T and its P
     uint32_t v_rd[DTW];
 #pragma unroll
@@ -210,12 +210,15 @@ __global__ void __launch_bounds__(kThreads, D == 256 ? 1 : (D == 128 && QK_INT8)
         float mx = -INFINITY;
         if (qk_wave) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float v = QK_INT8 ? (float)si[r] * kk[r >> 2][r & 3] : sf[r];
-                if (tail && 8 * (r >> 2) + (r & 3) >= key_lim) v = -INFINITY;
-                x[r] = v;
-                mx = fmaxf(mx, v);
+            for (int r = 0; r < 16; ++r) x[r] = QK_INT8 ? (float)si[r] * kk[r >> 2][r & 3] : sf[r];
+            if (tail) {
+                // (a branch of its own, kept one by the empty statement: see fwd_decode_full_int8_kernel)
+                asm volatile("");
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x[r] = hide_past(x[r], key_lim - 1, 8 * (r >> 2) + (r & 3));
             }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, x[r]);
             mx = half_pair_max(mx);
             if (lh == 0) *(float*)(smem + xm_wr) = mx;
         }

@@ -58,5 +58,7 @@ def scan(asm: str) -> List[str]:
             findings.append(f"{kernel}: line {n}: `{line.strip()}` stores while exec is narrowed (since line {narrowed_at})")
         if _BLOCK_END.match(line):
             close_block()
+            if line.split()[0] in ("s_endpgm", "s_setpc_b64"):
+                narrowed_at = 0          # nothing falls through: what follows is reached by branches, each with its own mask
     close_block()
     return findings

@@ -44,3 +44,13 @@ def test_spills_with_the_full_mask_and_scalar_branches_pass():
     ok = (HEAD + "\ts_and_saveexec_b64 s[2:3], vcc\n\ts_cbranch_execz .LBB0_2\n; %bb.1:\n\tv_mov_b32_e32 v5, 0\n"
           ".LBB0_2:\n\ts_or_b64 exec, exec, s[2:3]\n" + SPILL + RELOAD + "\ts_endpgm\n")
     assert spill_check.scan(ok) == []
+
+
+def test_a_mask_narrowed_ahead_of_the_program_end_does_not_reach_the_code_behind_it():
+    """A guarded store and `s_endpgm` close one path; the block behind it is entered by branches with their own mask."""
+    asm = (HEAD + "\ts_cbranch_scc1 .LBB0_3\n; %bb.1:\n\ts_and_b64 exec, exec, s[2:3]\n\ts_cbranch_execz .LBB0_2\n; %bb.4:\n"
+           "\tglobal_store_dword v[2:3], v1, off\n.LBB0_2:\n\ts_endpgm\n.LBB0_3:\n" + SPILL + RELOAD + "\ts_endpgm\n")
+    assert spill_check.scan(asm) == []
+    # ... while the same store on the fall-through side of the narrowing is still reported
+    bad = HEAD + "\ts_and_b64 exec, exec, s[2:3]\n" + SPILL + "\ts_endpgm\n"
+    assert any("while exec is narrowed" in f for f in spill_check.scan(bad))
