@@ -134,7 +134,7 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
     uint32_t v_rd[DTW];
 #pragma unroll
     for (int j = 0; j < DTW; ++j) {
-        const int dt = wave + 4 * j;
+        const int dt = (wave + 4 * j) % DT;          // (head_dim 64: waves 2 and 3 shadow tiles 0 and 1, see below)
         const int c = 2 * dt + (g16 & 1);
         v_rd[j] = OFF_V + v_row0 * D + 8 * (i16 & 1) + (((c & SWM) ^ v_swz) << 4) + ((c & ~SWM) << 4);
     }
@@ -146,7 +146,9 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
     const uint32_t xp_rd = OFF_XP + 16 * lane;                       // + 1024 per wave
     const uint32_t vs_wr = OFF_VS + 4 * (vs_thread ? vs_c : 0);
     const uint32_t vs_rd = OFF_VS + 16 * lh;                         // + 4 * (32*dt + 8*a4) per read
-    const bool own_tile0 = DT >= 4 || wave < DT;                     // head_dim 64: waves 2 and 3 own no output tile
+    // head_dim 64 has two output tiles for four waves: waves 2 and 3 compute tiles 0 and 1 a second time and store
+    // nothing (the same instruction stream for every wave; a run-time "owns a tile" test around the V fragments and the
+    // accumulator update costs the owners a hundred register copies per step)
     // the last visible key of the first row of this query block, and of the lane's row
     const int first_lim = p.causal ? (fold ? 0 : mb * kDecodeRows) + causal_off : 0x3fffffff;
     const int row_lim = p.causal ? (fold ? q_row % fold : q_row) + causal_off : 0x3fffffff;
@@ -181,7 +183,6 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
         for (int j = 0; j < DTW; ++j)
 #pragma unroll
             for (int st = 0; st < NST; ++st) {
-                if (j == 0 && !own_tile0) continue;        // head_dim 64: waves 2 and 3 own no output tile (and no V columns)
                 const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
                     (__attribute__((address_space(3))) v2i*)INTFA_LDS(smem + v_rd[j] + VB + (32 * st) * D));
                 const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
@@ -249,7 +250,7 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
             for (int j = 0; j < DTW; ++j)
 #pragma unroll
                 for (int a4 = 0; a4 < 4; ++a4)
-                    if (j > 0 || own_tile0) vsc[j][a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (32 * (wave + 4 * j) + 8 * a4));
+                    vsc[j][a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (32 * ((wave + 4 * j) % DT) + 8 * a4));
         }
         __syncthreads();                                   // the four P8 fragments are in LDS
         v4i pall[NST];
@@ -258,7 +259,6 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
         // -------- this wave's output columns: O^T[d, q] += V^T[d, key] P^T[key, q] over the whole block
 #pragma unroll
         for (int j = 0; j < DTW; ++j) {
-            if (j == 0 ? !own_tile0 : false) continue;
             if (NBS == 1) {
                 v16i acc = (v16i){0};
 #pragma unroll
