@@ -204,7 +204,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--workload", default="full_int8_B4_H32_N4096_d128", choices=sorted(WORKLOADS))
-    ap.add_argument("--p-round", default="rne", choices=["rne", "reference"])
+    ap.add_argument("--p-round", default="reference", choices=["rne", "reference"])
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU-baseline budget; 0 skips it")
     ap.add_argument("--no-parity", action="store_true", help="skip the oracle check of one head")
     ap.add_argument("--no-other-rounding", action="store_true",

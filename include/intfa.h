@@ -17,7 +17,9 @@
  *     synchronise, allocate or free;
  *   - return value: 0 on success, a negative INTFA_ERR_* for a rejected argument, a positive hipError_t when
  *     the launch itself failed;
- *   - re-entrant and thread-safe for distinct streams (no mutable global state).
+ *   - re-entrant and thread-safe for distinct streams: no mutable global state, with ONE exception -
+ *     intfa_fwd_full_int8_static keeps a per-device table of its scratch array's address and all its calls on one
+ *     GPU share that array (see its declaration).
  */
 #ifndef INTFA_H_
 #define INTFA_H_
@@ -29,7 +31,7 @@
 extern "C" {
 #endif
 
-#define INTFA_VERSION 7
+#define INTFA_VERSION 8
 
 /* forward variants (one entry point each, below) */
 enum { INTFA_VARIANT_FULL_INT8 = 0, INTFA_VARIANT_HALF_INT8 = 1, INTFA_VARIANT_FP16 = 2 };
@@ -39,10 +41,11 @@ enum { INTFA_F16 = 0, INTFA_BF16 = 1, INTFA_F32 = 2 };
 
 /* rounding used when P is requantised to int8 (full-int8 path) */
 enum {
-    /* 127*p evaluated in fp32 and rounded to nearest-even by one hardware convert */
-    INTFA_PROUND_RNE = 0,
-    /* the reference's fp16 sequence: fp16(p) * 127, + 0.5, truncating cast (flash_atten_full_int8.py:49-51) */
-    INTFA_PROUND_REFERENCE = 1
+    /* the reference's fp16 sequence: fp16(p) * 127, + 0.5, truncating cast (flash_atten_full_int8.py:49-51); the
+       default: what a zero-initialised parameter block selects */
+    INTFA_PROUND_REFERENCE = 0,
+    /* opt-in: 127*p evaluated in fp32 and rounded to nearest-even by one hardware convert */
+    INTFA_PROUND_RNE = 1
 };
 
 enum {
@@ -106,9 +109,11 @@ typedef struct intfa_fwd_params {
                                  are dealt evenly to the splits (ceil(blocks / num_splits) consecutive blocks each).  With
                                  causal the general kernels deal, per query block of 128 rows, the blocks VISIBLE to that
                                  query block (ceil(visible / num_splits) each, so no split of a query block is empty);
-                                 decode-shaped full-int8 calls (seqlen <= 64, head_dim <= 128) keep the partition of the
-                                 whole key sequence also with causal.  The requantisation frame of P depends on the
-                                 ranges, so a bit-faithful CPU evaluation must use the same ones. */
+                                 decode-shaped calls (seqlen <= 64; every variant and head_dim, except full-int8 at
+                                 head_dim 256 with blocked V scales, which runs the general kernel) keep the partition of
+                                 the whole key sequence also with causal: split s takes blocks s * ceil(blocks /
+                                 num_splits) onward, cut at the last visible block.  The requantisation frame of P depends
+                                 on the ranges, so a bit-faithful CPU evaluation must use the same ones. */
     void*   workspace;        /* device scratch of at least intfa_fwd_workspace_bytes() bytes, or NULL */
     size_t  workspace_bytes;
 

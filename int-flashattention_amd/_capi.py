@@ -11,9 +11,9 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libintfa.so")
 
-ABI_VERSION = 7          # INTFA_VERSION of include/intfa.h this mirror was written against
+ABI_VERSION = 8          # INTFA_VERSION of include/intfa.h this mirror was written against
 INTFA_F16, INTFA_BF16, INTFA_F32 = 0, 1, 2
-PROUND_RNE, PROUND_REFERENCE = 0, 1
+PROUND_REFERENCE, PROUND_RNE = 0, 1
 STATIC_SCRATCH_BYTES = 32 << 20      # INTFA_STATIC_SCRATCH_BYTES
 
 

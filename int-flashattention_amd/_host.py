@@ -55,7 +55,7 @@ def _require_gpu(*ts):
 
 
 def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: bool, sm_scale: float, out_dtype,
-                   num_splits: int = 1, p_round: int = _capi.PROUND_RNE, return_lse: bool = False,
+                   num_splits: int = 1, p_round: int = _capi.PROUND_REFERENCE, return_lse: bool = False,
                    v_scale_block: Optional[int] = None, seqlens_k: Optional[torch.Tensor] = None):
     lib = _capi.load()
     _require_gpu(q, k, v, q_scale, k_scale, v_scale)

@@ -39,11 +39,15 @@ def build_c_caller(verbose: bool = True) -> str:
     return C_CALLER
 
 
-def build(verbose: bool = True, jobs: int = 8) -> str:
+def build(verbose: bool = True, jobs: int = 8, only=None) -> str:
+    """Compiles every source and links the library.  `only` (development): a list of name fragments - sources whose file
+    name contains none of them keep their existing object file."""
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     srcs = sources()
     objs = [os.path.join(objdir, os.path.basename(s)[:-4] + ".o") for s in srcs]
+    todo = [(s, o) for s, o in zip(srcs, objs)
+            if not only or not os.path.exists(o) or any(frag in os.path.basename(s) for frag in only)]
 
     def compile_one(pair):
         # -save-temps=obj leaves the device assembly beside the object: it is scanned for register spills that lose lanes
@@ -69,7 +73,7 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
         return findings
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        findings = [x for fs in ex.map(compile_one, zip(srcs, objs)) for x in fs]
+        findings = [x for fs in ex.map(compile_one, todo) for x in fs]
     if findings:
         raise RuntimeError("the compiler placed register spills where lanes are masked off (wrong results for those lanes):\n  "
                            + "\n  ".join(findings[:20]))
@@ -77,12 +81,13 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
     if verbose:
-        print(f"built {OUT} from {len(srcs)} source file(s)")
+        print(f"built {OUT} from {len(srcs)} source file(s), {len(todo)} compiled")
     if os.path.exists(C_CALLER_SRC):
         build_c_caller(verbose)
     return OUT
 
 
 if __name__ == "__main__":
-    build()
+    # python -m int_flashattention_amd.build [--only fragment,fragment,...]
+    build(only=sys.argv[2].split(",") if len(sys.argv) > 2 and sys.argv[1] == "--only" else None)
     sys.exit(0)

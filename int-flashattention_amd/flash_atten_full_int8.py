@@ -6,7 +6,7 @@ from ._host import launch_forward
 
 
 def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, *, out_dtype=torch.float16,
-                        num_splits=1, p_round="rne", return_lse=False, v_scale_block=None, seqlens_k=None):
+                        num_splits=1, p_round="reference", return_lse=False, v_scale_block=None, seqlens_k=None):
     """Full-int8 attention forward.
 
     q, k, v: int8 [Z, H, N, d]; q_scale, k_scale: [Z, H, N] per-token scales; v_scale: [Z, H];
@@ -26,8 +26,8 @@ def attention_full_int8(q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, *,
     ``seqlens_k`` (int32 [Z] on the device): number of keys of each batch entry when k and v are a cache filled to
     different lengths; rows past an entry's length are not read.
 
-    ``p_round``: "rne" folds 127 into the exponent and rounds to nearest-even; "reference" reproduces the
-    fp16 sequence of flash_atten_full_int8.py:49-51.
+    ``p_round``: "reference" (the default) reproduces the fp16 sequence of flash_atten_full_int8.py:49-51 when P is
+    requantised; "rne" is an opt-in that folds 127 into the exponent and rounds to nearest-even in fp32.
     """
     pr = {"rne": _capi.PROUND_RNE, "reference": _capi.PROUND_REFERENCE}[p_round]
     return launch_forward("full", q, k, v, q_scale, k_scale, v_scale, causal, sm_scale, out_dtype,

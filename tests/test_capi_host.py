@@ -172,7 +172,7 @@ def test_entry_points_keep_the_reference_asserts():
         _host.check_head_dims(torch.zeros((1, 1, 128, 64)), torch.zeros((1, 1, 128, 32)), torch.zeros((1, 1, 128, 64)))
     q = torch.zeros((1, 1, 128, 64), dtype=torch.int8)
     with pytest.raises(RuntimeError, match="GPU only"):     # no CPU fallback
-        M.attention_full_int8(q, q, q, s, s, torch.ones((1, 1), dtype=torch.float16), False, 1.0)
+        M.attention_full_int8(q, q, q, s, s, torch.ones((1, 1), dtype=torch.float16), False, 1.0, p_round="rne")
 
 
 def test_split_count_heuristic():

@@ -37,7 +37,7 @@ def test_c_caller_output_equals_the_python_wrappers(tmp_path, Bz, H, N, D, causa
     got = torch.from_numpy(np.fromfile(fout, dtype=np.float16).reshape(Bz, H, N, D))
     dev = "cuda"
     want = M.attention_full_int8(q8.to(dev), k8.to(dev), v8.to(dev), qs.to(dev), ks.to(dev), vs.to(dev), causal, D ** -0.5,
-                                 num_splits=splits)
+                                 num_splits=splits, p_round="rne")
     torch.cuda.synchronize()
     assert torch.equal(got, want.cpu())
 

@@ -30,7 +30,7 @@ def _calls():
         sm = D ** -0.5
         t = [x.to(DEV) for x in (q, k, v, q8, qs, k8, ks, v8, vs)]
         q, k, v, q8, qs, k8, ks, v8, vs = t
-        out.append(lambda q8=q8, k8=k8, v8=v8, qs=qs, ks=ks, vs=vs, c=causal, sm=sm, s=splits: M.attention_full_int8(q8, k8, v8, qs, ks, vs, c, sm, num_splits=s))
+        out.append(lambda q8=q8, k8=k8, v8=v8, qs=qs, ks=ks, vs=vs, c=causal, sm=sm, s=splits: M.attention_full_int8(q8, k8, v8, qs, ks, vs, c, sm, num_splits=s, p_round="rne"))
         out.append(lambda q8=q8, k8=k8, v=v, qs=qs, ks=ks, c=causal, sm=sm, s=splits: M.attention_int8(q8, k8, v, qs, ks, c, sm, num_splits=s))
         out.append(lambda q=q, k=k, v=v, c=causal, sm=sm, s=splits: M.attention(q, k, v, c, sm, num_splits=s))
     return out

@@ -79,7 +79,7 @@ def test_decode_blocked_v_scales_bf16_and_strided_cache():
     vbig = torch.zeros((B, H_kv, 1024, D), dtype=torch.int8, device=DEV); vbig[:, :, :Nk] = x["v8"].to(DEV)
     q8, qs, ks, vs = gpu(x["q8"], x["qs"], x["ks"], x["vs"])
     o = M.attention_full_int8(q8, kbig[:, :, :Nk], vbig[:, :, :Nk], qs, ks, vs, False, sm, out_dtype=torch.bfloat16,
-                              v_scale_block=256)
+                              v_scale_block=256, p_round="rne")
     torch.cuda.synchronize()
     ref = oracle(x, sm, 128, p_requant=O.p_requant_rne, out_dtype=torch.bfloat16, v_scale_block=256)
     assert o.dtype == torch.bfloat16
@@ -93,8 +93,8 @@ def test_decode_kernel_agrees_with_the_general_kernel():
     sm = 128 ** -0.5
     k8, v8, ks, vs = gpu(x["k8"], x["v8"], x["ks"], x["vs"])
     q8, qs = gpu(x["q8"], x["qs"])
-    general = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm)
-    decode = M.attention_full_int8(q8[:, :, :64].contiguous(), k8, v8, qs[:, :, :64].contiguous(), ks, vs, False, sm)
+    general = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, p_round="rne")
+    decode = M.attention_full_int8(q8[:, :, :64].contiguous(), k8, v8, qs[:, :, :64].contiguous(), ks, vs, False, sm, p_round="rne")
     torch.cuda.synchronize()
     assert max_abs(decode, general[:, :, :64]) <= 1e-3 and mean_rel(decode, general[:, :, :64]) <= 1e-5
 
@@ -111,13 +111,13 @@ def test_decode_full_size_against_one_head_of_the_oracle():
     ks = (torch.rand((B, H, Nk), generator=g, device=DEV) * 0.01 + 0.02).half()
     vs = (torch.rand((B, H), generator=g, device=DEV) * 0.01 + 0.02).half()
     sm = D ** -0.5
-    o1 = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, num_splits="auto")
-    o2 = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, num_splits="auto")
+    o1 = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, num_splits="auto", p_round="rne")
+    o2 = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, num_splits="auto", p_round="rne")
     torch.cuda.synchronize()
     assert torch.equal(o1, o2)
     b, h = 5, 17
     c = lambda t: t[b:b + 1, h:h + 1].cpu()
-    single = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm)
+    single = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, p_round="rne")
     ref = O.attention_full_int8(c(q8), c(k8), c(v8), c(qs), c(ks), c(vs), False, sm, block_n=128, p_requant=O.p_requant_rne)
     assert max_abs(single[b:b + 1, h:h + 1], ref) <= 2e-3
     # the split pass quantises P per split (outputs here are of order one: compare in the mean-relative measure)
@@ -140,7 +140,7 @@ def test_per_batch_key_lengths_equal_sliced_calls(variant, Nq, D):
         c = lambda t: t[sel_b].to(DEV)
         if variant == "full":
             return M.attention_full_int8(c(x["q8"]), c(x["k8"])[:, :, :nk], c(x["v8"])[:, :, :nk], c(x["qs"]), c(x["ks"])[:, :, :nk],
-                                         c(x["vs"]), False, sm, return_lse=True, **kw)
+                                         c(x["vs"]), False, sm, return_lse=True, p_round="rne", **kw)
         if variant == "half":
             return M.attention_int8(c(x["q8"]), c(x["k8"])[:, :, :nk], c(x["v"])[:, :, :nk], c(x["qs"]), c(x["ks"])[:, :, :nk],
                                     False, sm, return_lse=True, **kw)
@@ -175,9 +175,9 @@ def test_per_batch_key_lengths_with_split_kv_and_argument_checks():
         assert max_abs(one[b:b + 1], ref) <= 4e-3
         assert max_abs(split[b:b + 1], ref) <= MAX_ABS and mean_rel(split[b:b + 1], ref) <= 3e-2
     with pytest.raises(ValueError):
-        M.attention_full_int8(*args, False, sm, seqlens_k=sl.long())
+        M.attention_full_int8(*args, False, sm, seqlens_k=sl.long(), p_round="rne")
     with pytest.raises(ValueError):
-        M.attention_full_int8(*args, False, sm, seqlens_k=sl[:2])
+        M.attention_full_int8(*args, False, sm, seqlens_k=sl[:2], p_round="rne")
 
 
 # ------------------------------------------------------------------------------------------ causal decode shapes
@@ -221,8 +221,8 @@ def test_causal_decode_with_split_kv_and_per_batch_lengths():
     sm = D ** -0.5
     sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
     args = gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"])
-    one = M.attention_full_int8(*args, True, sm, seqlens_k=sl)
-    split = M.attention_full_int8(*args, True, sm, seqlens_k=sl, num_splits=4)
+    one = M.attention_full_int8(*args, True, sm, seqlens_k=sl, p_round="rne")
+    split = M.attention_full_int8(*args, True, sm, seqlens_k=sl, num_splits=4, p_round="rne")
     torch.cuda.synchronize()
     for b, n in enumerate(lens):
         c = lambda t: t[b:b + 1]
@@ -232,19 +232,22 @@ def test_causal_decode_with_split_kv_and_per_batch_lengths():
         assert max_abs(split[b:b + 1], ref) <= MAX_ABS and mean_rel(split[b:b + 1], ref) <= 3e-2, (b, n)
 
 
+@pytest.mark.parametrize("D,v_block", [(128, 256), (256, None), (64, None)])
 @pytest.mark.parametrize("p_round,rq", [("reference", O.p_requant_reference), ("rne", O.p_requant_rne)])
-def test_causal_decode_split_matches_oracle_with_the_same_partition(p_round, rq):
-    """The decode kernel deals ceil(blocks / splits) key blocks to every split (csrc/flash_fwd_kernel.h:503) and applies
-    the causal mask inside them; the oracle evaluated over the same key ranges and merged by splitkv_combine must agree
-    to the rounding of the output (here also with blocked V scales and grouped heads)."""
-    B, H, H_kv, Nq, Nk, D, splits = 1, 8, 1, 64, 499, 128, 4
-    x = decode_inputs(B, H, H_kv, Nq, Nk, D, seed=100, v_block=256)
+def test_causal_decode_split_matches_oracle_with_the_same_partition(p_round, rq, D, v_block):
+    """Every decode-shaped call deals ceil(blocks / splits) key blocks of the WHOLE sequence to every split
+    (csrc/flash_fwd_kernel.h:503), blocks of the variant's own length (64 keys at head_dim 256 and 64), and applies the causal
+    mask inside them; the oracle evaluated over the same key ranges and merged by splitkv_combine must agree to the rounding
+    of the output (at head_dim 128 also with blocked V scales and grouped heads)."""
+    B, H, H_kv, Nq, Nk, splits = 1, 8, 1, 64, 499, 4
+    bn = M.block_n("full", D)
+    x = decode_inputs(B, H, H_kv, Nq, Nk, D, seed=100, v_block=v_block)
     sm = D ** -0.5
     o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), True, sm, num_splits=splits,
-                              p_round=p_round, v_scale_block=256)
+                              p_round=p_round, v_scale_block=v_block)
     torch.cuda.synchronize()
     rep = lambda t: t.repeat_interleave(H // H_kv, dim=1)
-    nblk = (Nk + 127) // 128
+    nblk = (Nk + bn - 1) // bn
     per = (nblk + splits - 1) // splits
     o_parts = torch.zeros((splits, B, H, Nq, D))
     lse_parts = torch.full((splits, B, H, Nq), float("-inf"))
@@ -253,7 +256,7 @@ def test_causal_decode_split_matches_oracle_with_the_same_partition(p_round, rq)
         if b0 >= b1:
             continue
         acc, l, m = O._blocked_forward("full", x["q8"], rep(x["k8"]), rep(x["v8"]), x["qs"], rep(x["ks"]), rep(x["vs"]), True, sm,
-                                       128, 128, key_lo=b0 * 128, key_hi=min(b1 * 128, Nk), p_requant=rq, v_scale_block=256)
+                                       128, bn, key_lo=b0 * bn, key_hi=min(b1 * bn, Nk), p_requant=rq, v_scale_block=v_block)
         seen = ~torch.isinf(m)
         o_parts[s] = torch.where(seen[..., None], acc / l[..., None], torch.zeros_like(acc))
         lse_parts[s] = torch.where(seen, m + torch.log2(l), torch.full_like(m, float("-inf")))
@@ -309,8 +312,8 @@ def test_decode_head_dim_256_agrees_with_the_general_kernel(causal):
     k8, v8, ks, vs = gpu(x["k8"], x["v8"], x["ks"], x["vs"])
     q8, qs = gpu(x["q8"], x["qs"])
     rows = slice(1, 65) if causal else slice(0, 64)          # the mask is aligned to the end of the cache
-    general = M.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm)
-    decode = M.attention_full_int8(q8[:, :, rows].contiguous(), k8, v8, qs[:, :, rows].contiguous(), ks, vs, causal, sm)
+    general = M.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, p_round="rne")
+    decode = M.attention_full_int8(q8[:, :, rows].contiguous(), k8, v8, qs[:, :, rows].contiguous(), ks, vs, causal, sm, p_round="rne")
     torch.cuda.synchronize()
     assert max_abs(decode, general[:, :, rows]) <= 1e-3 and mean_rel(decode, general[:, :, rows]) <= 1e-5
 
@@ -344,7 +347,7 @@ def test_decode_head_dim_256_per_batch_key_lengths(causal):
     def call(sel_b, nk, **kw):
         c = lambda t: t[sel_b].to(DEV)
         return M.attention_full_int8(c(x["q8"]), c(x["k8"])[:, :, :nk], c(x["v8"])[:, :, :nk], c(x["qs"]), c(x["ks"])[:, :, :nk],
-                                     c(x["vs"]), causal, sm, return_lse=True, **kw)
+                                     c(x["vs"]), causal, sm, return_lse=True, p_round="rne", **kw)
 
     o, lse = call(slice(None), Nk, seqlens_k=sl)
     torch.cuda.synchronize()
@@ -362,7 +365,7 @@ def test_decode_head_dim_256_blocked_v_scales_stay_with_the_general_kernel():
     B, H, Nq, Nk, D = 1, 2, 4, 600, 256
     x = decode_inputs(B, H, H, Nq, Nk, D, seed=114, v_block=128)
     sm = D ** -0.5
-    o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, sm, v_scale_block=128)
+    o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, sm, v_scale_block=128, p_round="rne")
     torch.cuda.synchronize()
     ref = oracle(x, sm, 64, p_requant=O.p_requant_rne, v_scale_block=128)
     assert max_abs(o, ref) <= 4e-3 and mean_rel(o, ref) <= 1e-3

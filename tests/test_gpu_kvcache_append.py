@@ -83,10 +83,10 @@ def test_cache_built_by_appends_decodes_like_the_quantised_concatenation():
         lens_d = lens_d + 1
         q = torch.randn((Z, H, 1, d), generator=g).half()
         q8, qs = M.quant_pertoken(q.to(DEV))
-        o = M.attention_full_int8(q8, kc, vc, qs, ksc, vs_d, False, sm, seqlens_k=lens_d)
+        o = M.attention_full_int8(q8, kc, vc, qs, ksc, vs_d, False, sm, seqlens_k=lens_d, p_round="rne")
         for b in range(Z):
             n = lens[b] + step + 1
             k8, ks = M.quant_pertoken(k[b:b + 1, :, :n].to(DEV))
             v8 = torch.round(v[b:b + 1, :, :n] / vs[b:b + 1, :, None, None]).clamp(-127, 127).to(torch.int8).to(DEV)
-            want = M.attention_full_int8(q8[b:b + 1], k8, v8, qs[b:b + 1], ks, vs_d[b:b + 1], False, sm)
+            want = M.attention_full_int8(q8[b:b + 1], k8, v8, qs[b:b + 1], ks, vs_d[b:b + 1], False, sm, p_round="rne")
             assert torch.equal(o[b:b + 1], want)

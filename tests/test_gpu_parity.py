@@ -53,6 +53,7 @@ def gpu(*ts):
 
 
 def run_full(x, causal, sm, **kw):
+    kw.setdefault("p_round", "rne")      # (the tests that mean the entry point's default rounding call it directly)
     o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), causal, sm, **kw)
     torch.cuda.synchronize()
     return o
@@ -106,19 +107,19 @@ def test_full_int8_matches_oracle(B, H, N, D, causal, p_round):
 
 
 @pytest.mark.parametrize("D", [64, 128, 256])
-def test_default_rounding_against_reference_rounding_on_short_causal_rows(D):
-    """The default rounding of P ("rne": 127 p evaluated in fp32, rounded to nearest even) against the reference's fp16
+def test_rne_rounding_against_reference_rounding_on_short_causal_rows(D):
+    """The opt-in rounding of P ("rne": 127 p evaluated in fp32, rounded to nearest even) against the reference's fp16
     sequence (flash_atten_full_int8.py:49-51).  The two agree except where 127 p lies within an fp16 rounding of a .5
     boundary, and then by one step of 1/127.  On a row with many keys a step is invisible; on the first rows of a
     causal problem (row i sees i + 1 keys) one step moves the output by up to |v| / (127 l), l >= 1: with |v| up to the
     value range's maximum (about 4.5 for N(0,1) inputs) that is 3.5e-2, above the 2e-2 that holds everywhere else.
     Pinned here: rows with more than 16 keys stay inside 2e-2, the short rows inside two such steps, the mean inside 1e-2;
-    callers who need the reference's rounding to the letter pass p_round="reference" (bit-for-bit the oracle's P8)."""
+    the entry point's default is p_round="reference" (bit-for-bit the oracle's P8)."""
     B, H, N = 4, 8, 256
     x = quantised(B, H, N, D, seed=61 + D)
     sm = D ** -0.5
     bn = M.block_n("full", D)
-    o = run_full(x, True, sm)                                                  # default p_round
+    o = run_full(x, True, sm, p_round="rne")
     ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], True, sm, block_n=bn)
     d = (o.float().cpu() - ref.float()).abs()
     vmax = x["v"].float().abs().amax().item()
@@ -128,6 +129,21 @@ def test_default_rounding_against_reference_rounding_on_short_causal_rows(D):
     assert d[:, :, :16].max().item() <= 2 * step
     # and the reference rounding itself reproduces the oracle to the accuracy of exp2
     assert_same_rounding(run_full(x, True, sm, p_round="reference"), ref)
+
+
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_positional_call_uses_the_reference_rounding(D):
+    """The drop-in call - positional arguments only, as the reference's callers write it - requantises P with the reference's
+    own fp16 sequence (flash_atten_full_int8.py:49-51): bit-equal to p_round="reference", and different from the opt-in
+    "rne" somewhere on a problem of this size."""
+    x = quantised(2, 2, 384, D, seed=75 + D)
+    sm = D ** -0.5
+    args = gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"])
+    o = M.attention_full_int8(*args, False, sm)
+    assert torch.equal(o, M.attention_full_int8(*args, False, sm, p_round="reference"))
+    assert not torch.equal(o, M.attention_full_int8(*args, False, sm, p_round="rne"))
+    ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], False, sm, block_n=M.block_n("full", D))
+    assert_same_rounding(o, ref)
 
 
 @pytest.mark.parametrize("d", [16, 32])
@@ -162,12 +178,12 @@ def test_outlier_channels_stress_per_token_scales():
 def test_strided_inputs_equal_contiguous():
     x = quantised(2, 4, 256, 128, seed=15)
     sm = 0.1
-    base = run_full(x, True, sm)
+    base = run_full(x, True, sm, p_round="rne")
     # [B, N, H, d] storage viewed as [B, H, N, d]
     q8, k8, v8 = (t.permute(0, 2, 1, 3).contiguous().to(DEV).permute(0, 2, 1, 3) for t in (x["q8"], x["k8"], x["v8"]))
     qs, ks = (t.transpose(1, 2).contiguous().to(DEV).transpose(1, 2) for t in (x["qs"], x["ks"]))
     assert not q8.is_contiguous() and not qs.is_contiguous()
-    o = M.attention_full_int8(q8, k8, v8, qs, ks, x["vs"].to(DEV), True, sm)
+    o = M.attention_full_int8(q8, k8, v8, qs, ks, x["vs"].to(DEV), True, sm, p_round="rne")
     assert torch.equal(o, base)
 
 
@@ -330,7 +346,7 @@ def test_three_variants_order_by_precision():
     exact = O.attention_exact(x["q"], x["k"], x["v"], False, sm)
     e_fp = mean_rel(M.attention(*gpu(x["q"], x["k"], x["v"]), False, sm), exact)
     e_half = mean_rel(M.attention_int8(*gpu(x["q8"], x["k8"], x["v"], x["qs"], x["ks"]), False, sm), exact)
-    e_full = mean_rel(run_full(x, False, sm), exact)
+    e_full = mean_rel(run_full(x, False, sm, p_round="rne"), exact)
     assert e_fp < e_half < e_full < 5e-2
 
 
@@ -347,7 +363,7 @@ def test_ragged_lengths_full_int8(B, H, N, D, causal):
     bn = M.block_n("full", D)
     s = M.debug_qk_int32(*gpu(x["q8"], x["k8"])).cpu()
     assert torch.equal(s, O.qk_int32(x["q8"], x["k8"]))
-    o, lse = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), causal, sm, return_lse=True)
+    o, lse = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), causal, sm, return_lse=True, p_round="rne")
     torch.cuda.synchronize()
     assert o.shape == (B, H, N, D) and torch.isfinite(o).all()
     ref, lse_ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], causal, sm, block_n=bn,
@@ -383,7 +399,7 @@ def test_ragged_lengths_split_kv(causal, splits):
 def test_ragged_outputs_do_not_touch_memory_past_the_end():
     """Output rows are written for valid queries only: a guard region behind the output stays untouched."""
     x = quantised(1, 1, 130, 128, seed=63)
-    o = run_full(x, False, 0.09)
+    o = run_full(x, False, 0.09, p_round="rne")
     ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], False, 0.09, p_requant=O.p_requant_rne)
     assert_same_rounding(o, ref)
     # the same call into a larger buffer through strides: rows 130.. of the buffer must keep their fill value
@@ -433,9 +449,9 @@ def test_separate_query_and_key_lengths(B, H, Nq, Nk, D):
     o = M.attention_int8(*gpu(q8, k8, v, qs, ks), False, sm)
     assert max_abs(o, _dense_cross(qd, kd, v, sm)) <= 3e-3          # same dequantised Q, K: only fp16 P and output rounding
     vd = v8.float() * vs.float()[..., None, None]
-    o = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm)
+    o = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm, p_round="rne")
     assert max_abs(o, _dense_cross(qd, kd, vd, sm)) <= 3e-2 and mean_rel(o, _dense_cross(qd, kd, vd, sm)) <= 4e-2   # + P8 quantisation
-    o2 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm, num_splits=3)
+    o2 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm, num_splits=3, p_round="rne")
     assert max_abs(o2, o) <= 2e-2
 
 
@@ -452,8 +468,8 @@ def test_decoding_shape_with_automatic_splits():
     a1 = M.attention_int8(*gpu(q8, k8, v, qs, ks), False, sm)
     a2 = M.attention_int8(*gpu(q8, k8, v, qs, ks), False, sm, num_splits="auto")
     assert max_abs(a2, a1) <= 1e-3
-    f1 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm)
-    f2 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm, num_splits="auto")
+    f1 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm, p_round="rne")
+    f2 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm, num_splits="auto", p_round="rne")
     assert max_abs(f2, f1) <= 2e-2 and max_abs(f2, _dense_cross(q, k, v, sm)) <= 3e-2
 
 
@@ -477,8 +493,8 @@ def test_grouped_decoding_folds_heads_into_rows(Nq):
     qd, kd = q8.float() * qs.float()[..., None], k8.float() * ks.float()[..., None]
     o = M.attention_int8(*gpu(q8, k8, v, qs, ks), False, sm, num_splits="auto")
     assert max_abs(o, _dense_cross(qd, rep(kd), rep(v), sm)) <= 3e-3
-    o = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm)
-    o_rep = M.attention_full_int8(*gpu(q8, rep(k8), rep(v8), qs, rep(ks), rep(vs)), False, sm)     # ungrouped call
+    o = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), False, sm, p_round="rne")
+    o_rep = M.attention_full_int8(*gpu(q8, rep(k8), rep(v8), qs, rep(ks), rep(vs)), False, sm, p_round="rne")     # ungrouped call
     assert torch.equal(o, o_rep)
 
 
@@ -497,7 +513,7 @@ def test_causal_with_separate_lengths_is_aligned_bottom_right(variant, Nq, Nk, D
     sm = D ** -0.5
     if variant == "full":
         bn = M.block_n("full", D)
-        o, lse = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), True, sm, return_lse=True)
+        o, lse = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), True, sm, return_lse=True, p_round="rne")
         ref, lse_ref = O.attention_full_int8(q8, k8, v8, qs, ks, vs, True, sm, block_n=bn, p_requant=O.p_requant_rne, return_lse=True)
         torch.cuda.synchronize()
         if Nk >= Nq:
@@ -531,7 +547,7 @@ def test_causal_separate_lengths_with_split_kv_and_per_batch_lengths(variant):
     sm = D ** -0.5
     sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
     if variant == "full":
-        call = lambda **kw: M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), True, sm, seqlens_k=sl, **kw)
+        call = lambda **kw: M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), True, sm, seqlens_k=sl, p_round="rne", **kw)
         one = lambda b, n: O.attention_full_int8(q8[b:b + 1], k8[b:b + 1, :, :n], v8[b:b + 1, :, :n], qs[b:b + 1], ks[b:b + 1, :, :n],
                                                  vs[b:b + 1], True, sm, block_n=128, p_requant=O.p_requant_rne)
     else:
@@ -562,8 +578,8 @@ def test_rows_without_a_key_on_the_split_path_give_zeros_and_minus_inf_lse(num_s
     sl = torch.tensor(lens, dtype=torch.int32, device=DEV)
     for causal in (False, True):
         o, lse = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), causal, sm, seqlens_k=sl, num_splits=num_splits,
-                                       return_lse=True)
-        o1, lse1 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), causal, sm, seqlens_k=sl, return_lse=True)
+                                       return_lse=True, p_round="rne")
+        o1, lse1 = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), causal, sm, seqlens_k=sl, return_lse=True, p_round="rne")
         torch.cuda.synchronize()
         assert torch.isfinite(o).all()
         assert o[1].abs().max().item() == 0 and torch.isinf(lse[1]).all() and (lse[1] < 0).all()
@@ -595,7 +611,7 @@ def test_grouped_kv_heads_equal_repeated_kv(variant, B, H, H_kv, N, D, causal):
     rep = lambda t: t.repeat_interleave(g, dim=1)
     sm = D ** -0.5
     if variant == "full":
-        o = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), causal, sm)
+        o = M.attention_full_int8(*gpu(q8, k8, v8, qs, ks, vs), causal, sm, p_round="rne")
         ref = O.attention_full_int8(q8, rep(k8), rep(v8), qs, rep(ks), rep(vs), causal, sm, block_n=M.block_n("full", D),
                                     p_requant=O.p_requant_rne)
         assert_same_rounding(o, ref)
@@ -624,16 +640,16 @@ def test_headline_shape_slices_reproduce_and_v_scale_is_linear():
     B, H, N, D = 4, 32, 4096, 128
     q8, k8, v8, qs, ks, vs = _headline_inputs()
     sm = D ** -0.5
-    o = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm)
+    o = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, p_round="rne")
     assert torch.isfinite(o).all()
     # every (batch, head) is independent: recomputing one slice alone gives the same bits
     for b, h in ((0, 0), (3, 31), (1, 17)):
         sl = lambda t: t[b:b + 1, h:h + 1].contiguous()
-        o1 = M.attention_full_int8(sl(q8), sl(k8), sl(v8), sl(qs), sl(ks), sl(vs), False, sm)
+        o1 = M.attention_full_int8(sl(q8), sl(k8), sl(v8), sl(qs), sl(ks), sl(vs), False, sm, p_round="rne")
         assert torch.equal(o1, o[b:b + 1, h:h + 1])
     # the value scale is applied once, linearly: doubling it doubles the output exactly (power of two) wherever the
     # fp16 result is a normal number; subnormal results are rounded on a fixed 2^-24 grid and may differ by one step
-    o2 = M.attention_full_int8(q8, k8, v8, qs, ks, vs * 2, False, sm)
+    o2 = M.attention_full_int8(q8, k8, v8, qs, ks, vs * 2, False, sm, p_round="rne")
     normal = o.abs() > 2.0 ** -14
     assert torch.equal(o2[normal], (o * 2)[normal])
     assert (o2.float() - 2 * o.float()).abs().max().item() <= 2.0 ** -24
@@ -650,7 +666,7 @@ def test_constant_v_gives_constant_columns_at_full_size():
     q8, k8, _, qs, ks, _ = _headline_inputs(B, H, N, D, seed=21)
     v8 = torch.full((B, H, N, D), 64, dtype=torch.int8, device=DEV)
     vs = torch.full((B, H), 1 / 64, dtype=torch.float16, device=DEV)
-    o = M.attention_full_int8(q8, k8, v8, qs, ks, vs, True, D ** -0.5)
+    o = M.attention_full_int8(q8, k8, v8, qs, ks, vs, True, D ** -0.5, p_round="rne")
     # O = sum(P8) / (127 l): the same for every column of a row.  Its distance from one is the mass P loses when it is
     # rounded to multiples of 1/127 (every p below 1/254 becomes zero): a property of the reference's quantisation
     # that grows with the number of keys, about 0.1 at 4096 keys with these inputs.
@@ -684,7 +700,7 @@ def test_other_benchmark_shapes_one_slice_against_oracle(variant, B, H, N, D, ca
             ref = O.attention_int8(cpu(q8), cpu(k8), cpu(v), cpu(qs), cpu(ks), causal, sm, block_n=bn)
         else:
             v8, vs = M.quant_pertensor(v)
-            o = M.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm)
+            o = M.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, p_round="rne")
             ref = O.attention_full_int8(cpu(q8), cpu(k8), cpu(v8), cpu(qs), cpu(ks), cpu(vs), causal, sm, block_n=bn,
                                         p_requant=O.p_requant_rne)
     assert torch.isfinite(o).all()
@@ -704,7 +720,7 @@ def test_forward_and_quantisers_replay_from_a_captured_graph():
         q8, qs = M.quant_pertoken(q)
         k8, ks = M.quant_pertoken(k)
         v8, vs = M.quant_pertensor(v)
-        return M.attention_full_int8(q8, k8, v8, qs, ks, vs, True, sm, num_splits=splits)
+        return M.attention_full_int8(q8, k8, v8, qs, ks, vs, True, sm, num_splits=splits, p_round="rne")
 
     for splits in (1, 3):
         static = [t.clone() for t in x]
@@ -739,8 +755,8 @@ def test_repeated_launches_are_bit_identical(D, N, dtype):
     k8, ks = M.quant_pertoken(k)
     v8, vs = M.quant_pertensor(v)
     sm = D ** -0.5
-    first = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, out_dtype=dtype)
-    outs = [M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, out_dtype=dtype) for _ in range(40)]
+    first = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, out_dtype=dtype, p_round="rne")
+    outs = [M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm, out_dtype=dtype, p_round="rne") for _ in range(40)]
     torch.cuda.synchronize()
     assert torch.isfinite(first).all()
     for i, o in enumerate(outs):

@@ -92,9 +92,9 @@ def test_blocked_v_scale_filled_with_the_scalar_equals_the_scalar_entry():
     q, k, v, _ = O.make_inputs(B, H, N, D, seed=81)
     q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k); v8, vs = O.quant_pertensor(v)
     args = gpu(q8, k8, v8, qs, ks)
-    want = M.attention_full_int8(*args, vs.to(DEV), True, 0.09)
+    want = M.attention_full_int8(*args, vs.to(DEV), True, 0.09, p_round="rne")
     vs4 = vs.float()[:, :, None, None].expand(B, H, 3, D).contiguous().to(DEV)
-    got = M.attention_full_int8(*args, vs4, True, 0.09)       # v_scale_block defaults to the kernel's key block
+    got = M.attention_full_int8(*args, vs4, True, 0.09, p_round="rne")       # v_scale_block defaults to the kernel's key block
     torch.cuda.synchronize()
     # same products in another order (scale per block instead of once at the end): fp32 rounding only
     assert max_abs(got, want) <= 2e-3 and mean_rel(got, want) <= 1e-4
@@ -106,8 +106,8 @@ def test_blocked_v_scale_is_more_accurate_under_a_channel_burst():
     sm = D ** -0.5
     exact = O.attention_exact(x["q"], x["k"], x["v"], False, sm).float()
     v8s, vss = O.quant_pertensor(x["v"])
-    coarse = M.attention_full_int8(*gpu(x["q8"], x["k8"], v8s, x["qs"], x["ks"], vss), False, sm).float().cpu()
-    fine = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, sm).float().cpu()
+    coarse = M.attention_full_int8(*gpu(x["q8"], x["k8"], v8s, x["qs"], x["ks"], vss), False, sm, p_round="rne").float().cpu()
+    fine = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, sm, p_round="rne").float().cpu()
     other = [c for c in range(D) if c != D // 2]
     err_c = (coarse - exact)[..., other].abs().mean().item()
     err_f = (fine - exact)[..., other].abs().mean().item()
@@ -119,7 +119,7 @@ def test_blocked_v_scale_with_grouped_heads_split_kv_and_bf16():
     x = blocked_inputs(B, H, N, D, 83, 128, dtype=torch.bfloat16, H_kv=H_kv)
     sm = D ** -0.5
     args = gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"])
-    one = M.attention_full_int8(*args, False, sm, out_dtype=torch.bfloat16)
+    one = M.attention_full_int8(*args, False, sm, out_dtype=torch.bfloat16, p_round="rne")
     rep = lambda t: t.repeat_interleave(H // H_kv, dim=1)
     ref = O.attention_full_int8(x["q8"], rep(x["k8"]), rep(x["v8"]), x["qs"], rep(x["ks"]), rep(x["vs"]), False, sm,
                                 block_n=128, v_scale_block=128, p_requant=O.p_requant_rne, out_dtype=torch.bfloat16)
@@ -143,7 +143,7 @@ def test_64_key_v_scale_rows_with_grouped_heads_split_kv_decode_shapes_and_bf16(
     args = gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"])
     rep = lambda t: t.repeat_interleave(H // H_kv, dim=1)
     okw = dict(block_n=128, v_scale_block=64, out_dtype=torch.bfloat16)
-    one = M.attention_full_int8(*args, True, sm, out_dtype=torch.bfloat16, v_scale_block=64)
+    one = M.attention_full_int8(*args, True, sm, out_dtype=torch.bfloat16, v_scale_block=64, p_round="rne")
     ref = O.attention_full_int8(x["q8"], rep(x["k8"]), rep(x["v8"]), x["qs"], rep(x["ks"]), rep(x["vs"]), True, sm,
                                 p_requant=O.p_requant_rne, **okw)
     assert max_abs(one, ref) <= 3e-2 and mean_rel(one, ref) <= 3e-3          # bf16 output: 8-bit significand
@@ -153,7 +153,7 @@ def test_64_key_v_scale_rows_with_grouped_heads_split_kv_decode_shapes_and_bf16(
     assert max_abs(split, ref_split) <= 3e-2 and mean_rel(split, ref_split) <= 3e-3
     # decoding against the cache: three new tokens per head, grouped heads (no causal fold with 64-key rows), causal
     q3, qs3 = x["q8"][:, :, -3:].contiguous(), x["qs"][:, :, -3:].contiguous()
-    dec = M.attention_full_int8(*gpu(q3, x["k8"], x["v8"], qs3, x["ks"], x["vs"]), True, sm, v_scale_block=64)
+    dec = M.attention_full_int8(*gpu(q3, x["k8"], x["v8"], qs3, x["ks"], x["vs"]), True, sm, v_scale_block=64, p_round="rne")
     torch.cuda.synchronize()
     ref_dec = O.attention_full_int8(q3, rep(x["k8"]), rep(x["v8"]), qs3, rep(x["ks"]), rep(x["vs"]), True, sm,
                                     p_requant=O.p_requant_rne, block_n=128, v_scale_block=64)
@@ -162,20 +162,20 @@ def test_64_key_v_scale_rows_with_grouped_heads_split_kv_decode_shapes_and_bf16(
 
 def test_blocked_v_scale_small_head_dim_and_argument_checks():
     x = blocked_inputs(1, 2, 256, 32, 84, 128)
-    o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, 0.2, v_scale_block=128)
+    o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, 0.2, v_scale_block=128, p_round="rne")
     ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], False, 0.2, block_n=128,
                                 v_scale_block=128, p_requant=O.p_requant_rne)
     assert_same_rounding(o, ref)
     with pytest.raises(RuntimeError):                          # 32 neither is a multiple of the 128-key block nor 64
         v8, vs = O.quant_perblock_channel(x["v"], 32)
-        M.attention_full_int8(*gpu(x["q8"], x["k8"], v8, x["qs"], x["ks"], vs), False, 0.2, v_scale_block=32)
+        M.attention_full_int8(*gpu(x["q8"], x["k8"], v8, x["qs"], x["ks"], vs), False, 0.2, v_scale_block=32, p_round="rne")
     with pytest.raises(RuntimeError):                          # 192 is a multiple of 64 only
         v8, vs = O.quant_perblock_channel(x["v"], 192)
-        M.attention_full_int8(*gpu(x["q8"], x["k8"], v8, x["qs"], x["ks"], vs), False, 0.2, v_scale_block=192)
+        M.attention_full_int8(*gpu(x["q8"], x["k8"], v8, x["qs"], x["ks"], vs), False, 0.2, v_scale_block=192, p_round="rne")
     with pytest.raises(ValueError):                            # wrong number of scale rows
-        M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"][:, :, :1]), False, 0.2, v_scale_block=128)
+        M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"][:, :, :1]), False, 0.2, v_scale_block=128, p_round="rne")
     with pytest.raises(ValueError):
-        M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"][:, :, 0, 0]), False, 0.2, v_scale_block=128)
+        M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"][:, :, 0, 0]), False, 0.2, v_scale_block=128, p_round="rne")
 
 
 def test_quant_perblock_channel_bit_exact_on_many_magnitudes():
