@@ -70,6 +70,13 @@ WORKLOADS = {
                                              dtype="bfloat16", std=0.5),
     "full_int8_B16_H16_N1024_d256_bf16": dict(variant="full", B=16, H=16, N=1024, D=256, causal=False, splits=1,
                                               dtype="bfloat16", std=0.5),
+    # the grid of the reference's own benchmark script (benchmark.py:23-45: BATCH, N_HEADS, HEAD_DIM = 4, 32, 64, N_CTX = 2^10 ..
+    # 2^14, non-causal, providers full-int8 / int8 / fp16), with this build's input recipe
+    "full_int8_B4_H32_N1024_d64": dict(variant="full", B=4, H=32, N=1024, D=64, causal=False, splits=1),
+    "full_int8_B4_H32_N4096_d64": dict(variant="full", B=4, H=32, N=4096, D=64, causal=False, splits=1),
+    "full_int8_B4_H32_N16384_d64": dict(variant="full", B=4, H=32, N=16384, D=64, causal=False, splits=1),
+    "half_int8_B4_H32_N4096_d64": dict(variant="half", B=4, H=32, N=4096, D=64, causal=False, splits=1),
+    "fp16_B4_H32_N4096_d64": dict(variant="fp", B=4, H=32, N=4096, D=64, causal=False, splits=1),
     # head_dim 256 at the headline's batch, heads and length (the eight-wave kernel of that head_dim)
     "full_int8_B4_H32_N4096_d256": dict(variant="full", B=4, H=32, N=4096, D=256, causal=False, splits=1),
     # the headline shape with V quantised per block of 128 keys and channel (the V scales of the reference's CUDA kernel)
@@ -135,7 +142,7 @@ def cpu_baseline(budget_s: float, w: dict):
     else:
         q8, qs = O.quant_pertoken(q); k8, ks = O.quant_pertoken(k)
         if variant == "full":
-            bn = 128 if D <= 128 else 64
+            bn = 128 if D == 128 else 64      # the kernels' key blocks (intfa_fwd_block_n)
             v_block = w.get("v_block")
             v8, vs = O.quant_perblock_channel(v, v_block) if v_block else O.quant_pertensor(v)
             kw = dict(v_scale_block=v_block) if v_block else {}

@@ -124,7 +124,7 @@ def launch_forward(variant: str, q, k, v, q_scale, k_scale, v_scale, causal: boo
     # so that a group streams its K/V once instead of g times.  Pure re-striding: same memory, same results per row.
     g = H // H_kv
     # (with the causal mask only where the kernel can be told the position of a row: the decode-shaped calls)
-    decode_kernel = (dk <= 128 and p.v_scale_block != 64) or (dk == 256 and p.v_scale_block == 0)
+    decode_kernel = not (dk == 128 and p.v_scale_block == 64)     # (64-key scale rows under the 128-key block: general kernel)
     fold_rows = 2 * BLOCK if not causal else (64 if decode_kernel else 0)
     if g > 1 and g * N <= fold_rows and _can_fold(q_, N) and (variant == "fp" or _can_fold(q_scale, N)):
         if causal:

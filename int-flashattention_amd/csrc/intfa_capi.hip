@@ -39,10 +39,11 @@ constexpr int kMaxSplits = 64;
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Key-block length of a variant at a head_dim: the full-int8 kernel takes 128 keys per block (64 at head_dim 256),
-// the kernels with a 16-bit P V take 64.
+// Key-block length of a variant at a head_dim.  Full-int8: 128 keys at head_dim 128, 64 at head_dim 64 (the reference
+// admits no key block longer than head_dim: tl.static_assert(BLOCK_N <= HEAD_DIM), flash_atten_full_int8.py:88) and at
+// head_dim 256 (registers and LDS); the kernels with a 16-bit P V take 64.
 int block_n_for(int variant, int head_dim) {
-    if (variant == INTFA_VARIANT_FULL_INT8) return head_dim <= 128 ? 128 : 64;
+    if (variant == INTFA_VARIANT_FULL_INT8) return head_dim == 128 ? 128 : 64;
     return 64;
 }
 
@@ -152,12 +153,8 @@ int launch_combine(const intfa_fwd_params* p, const KParams& kp, hipStream_t str
 
 // Few query rows per head (decoding against a cache): the pass runs a kernel whose waves share the keys of a block
 // instead of each taking 32 query rows (intfa_fwd_decode.h, intfa_fwd_decode_f16pv.h).
-// (Head_dim 256 of the full-int8 variant with blocked V scales stays with the general kernel.)
 constexpr int kDecodeMaxRows = 2 * kDecodeRows;
-bool decode_shaped(int variant, int seqlen, int head_dim, bool blocked_v_scales) {
-    if (seqlen > kDecodeMaxRows) return false;
-    return head_dim <= 128 || !(variant == INTFA_VARIANT_FULL_INT8 && blocked_v_scales);
-}
+bool decode_shaped(int seqlen) { return seqlen <= kDecodeMaxRows; }
 
 int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dump_s, hipStream_t stream) {
     const bool vblk = variant == INTFA_VARIANT_FULL_INT8 && !dump_s && kp.vs_g > 0;
@@ -169,9 +166,8 @@ int dispatch(int variant, const intfa_fwd_params* p, const KParams& kp, bool dum
     sel.dump_s = dump_s;
     const int d = kp.head_dim;
     if (vblk && kp.vs_sub == 2) {              // (also for few query rows: the decode kernel has one scale row per block)
-        if (d == 64) return launch_full_int8_vblk64_d64(kp, sel, stream);
         if (d == 128) return launch_full_int8_vblk64_d128(kp, sel, stream);
-    } else if (!dump_s && decode_shaped(variant, kp.seqlen, d, vblk)) {
+    } else if (!dump_s && decode_shaped(kp.seqlen)) {
         if (variant == INTFA_VARIANT_FULL_INT8) {
             if (d == 64) return launch_decode_full_int8_d64(kp, sel, stream);
             if (d == 128) return launch_decode_full_int8_d128(kp, sel, stream);
@@ -211,7 +207,7 @@ int run_forward(int variant, const intfa_fwd_params* p, int qk_bytes, int v_byte
     if (rc != INTFA_OK) return rc;
     if (variant == INTFA_VARIANT_FULL_INT8 && p->p_round != INTFA_PROUND_RNE && p->p_round != INTFA_PROUND_REFERENCE) return INTFA_ERR_DTYPE;
     if (p->causal_rows != 0) {
-        if (p->causal_rows < 0 || !p->causal || !decode_shaped(variant, kp.seqlen, kp.head_dim, kp.vs_g > 0) ||
+        if (p->causal_rows < 0 || !p->causal || !decode_shaped(kp.seqlen) ||
             kp.seqlen % p->causal_rows != 0 || kp.vs_sub == 2) return INTFA_ERR_SEQLEN;
         kp.causal_rows = p->causal_rows;
     }
@@ -246,7 +242,7 @@ const char* intfa_error_string(int code) {
         case INTFA_ERR_WORKSPACE: return "workspace missing, misaligned or too small for num_splits";
         case INTFA_ERR_SHAPE: return "batch and heads must be positive and the grid must fit 31 bits";
         case INTFA_ERR_SPLITS: return "num_splits must be at most 64";
-        case INTFA_ERR_VSCALE: return "v_scale_block must be a multiple of the key-block length (or 64 at head_dim <= 128) and vs_stride_blk at least head_dim";
+        case INTFA_ERR_VSCALE: return "v_scale_block must be a multiple of the key-block length (or 64 at head_dim 128) and vs_stride_blk at least head_dim";
         case INTFA_ERR_SCRATCH: return "the split-KV partials of this call exceed INTFA_STATIC_SCRATCH_BYTES (or the device index exceeds 63)";
         default: return code > 0 ? "hip error" : "unknown error";
     }
@@ -263,7 +259,7 @@ int intfa_fwd_suggest_splits(const intfa_fwd_params* p, int variant, int num_cus
     const int cus = num_cus > 0 ? num_cus : 256;
     int64_t slots = 2ll * cus;                                                 // two workgroups per compute unit
     int64_t wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kBlockM - 1) / kBlockM);
-    if (decode_shaped(variant, p->seqlen, p->head_dim, variant == INTFA_VARIANT_FULL_INT8 && p->v_scale_block > 0)) {
+    if (decode_shaped(p->seqlen)) {
         wgs = (int64_t)p->batch * p->heads * ((p->seqlen + kDecodeRows - 1) / kDecodeRows);
         // head_dim 256: 96 KiB and more of tiles, one workgroup per compute unit
         if (p->head_dim == 256) slots = cus;

@@ -39,17 +39,6 @@ template <bool V> struct BoolTag { static constexpr bool value = V; };
 constexpr int kBlockM = 128;
 constexpr int kThreads = 256;
 constexpr float kLog2_127 = 6.98868468677f;   // log2(127)
-// An int32 accumulator that starts from the bit pattern of 1.5 * 2^23 instead of 0 holds, for any sum |s| < 2^22, the bit
-// pattern of the fp32 number 1.5 * 2^23 + s exactly (unit in the last place 1 over that whole range).  The int8 dot
-// products of these kernels stay below 2^22 (127 * 127 * 256 for Q K^T at head_dim 256, 127 * 127 * 128 for P V), so
-// float(s) = as_float(acc) - kMagicF with no rounding, and s * c = fma(as_float(acc), c, -kMagicF * c) with the one
-// rounding of the product whenever kMagicF * c is exact (c with at most 22 significant bits: every fp16 / bf16 scale).
-constexpr int kMagicI = 0x4B400000;
-constexpr float kMagicF = 12582912.f;
-// Reinterprets an int32 accumulator register as fp32.  Always through this by-value helper: __builtin_bit_cast applied
-// directly to an element of an ext_vector (acc[r]) reads element 0 whatever r is (clang 22 of ROCm 7.2).
-__device__ __forceinline__ float as_f32(int x) { return __builtin_bit_cast(float, x); }
-
 // floor(n / d) for 0 <= n < 2^31 and a divisor d fixed per launch: (n * m) >> s with s = 31 + ceil(log2 d) and
 // m = ceil(2^s / d) < 2^32 computed on the host (Granlund & Montgomery, "Division by invariant integers using
 // multiplication").  For a wave-uniform n that is three scalar instructions; a run-time integer division expands to some

@@ -13,7 +13,8 @@
 // The int32 sums run over the same 128 keys as in the general kernel, so results agree with it up to the order of the
 // fp32 additions of the row sums.  K/V tiles are double-buffered in LDS and the whole next tile is requested at the
 // start of a block (the data comes from HBM, not from a cache shared with other query blocks).
-// Head_dim 256: the general kernel's key block is 64 there (fwd_full_int8_pair_kernel), so a 128-key step of this
+// Head dims 64 and 256: the general kernels' key block is 64 there (the reference admits no key block longer than head_dim,
+// flash_atten_full_int8.py:88; at 256 registers set the limit), so a 128-key step of this
 // kernel covers TWO blocks A (waves 0, 1) and B (waves 2, 3): after the one exchange of partial maxima every wave knows
 // m_A = max(m, max_A), m_B = max(m_A, max_B) and both factors alpha_A = 2^(m - m_A), alpha_B = 2^(m_A - m_B); each wave
 // requantises its keys in its own block's frame, and an output tile is updated as
@@ -24,17 +25,16 @@
 
 namespace intfa {
 
-// Head dims 64 and 128 (the key block of the general kernel is 128 there too, so both kernels evaluate the same blocks)
-// and 256 (two 64-key blocks per step; one scale per (batch, head) only).
+// Head_dim 128: one 128-key block per step, the block of the general kernel.  Head dims 64 and 256: two 64-key blocks.
 template <int D, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool SPLIT, bool VBLK>
 __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_int8_kernel(const KParams p) {
-    static_assert(D == 64 || D == 128 || (D == 256 && !VBLK), "head dims 64, 128, and 256 without blocked V scales");
+    static_assert(D == 64 || D == 128 || D == 256, "head dims 64, 128, 256");
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T
     constexpr int DT = D / 32;                   // 32-wide output tiles along head_dim; wave w owns tiles w, w+4, ...
     constexpr int DTW = (DT + 3) / 4;            // output tiles per wave
     constexpr int NST = 4, BN = 32 * NST;        // one 32-key sub-tile per wave
-    constexpr int NBS = D == 256 ? 2 : 1;        // key blocks (of the arithmetic) per step
+    constexpr int NBS = D == 128 ? 1 : 2;        // key blocks (of the arithmetic) per step
     constexpr int BNB = BN / NBS;                // key block of the arithmetic: intfa_fwd_block_n()
     constexpr int KT = BN * D, VT = BN * D;      // bytes of one K / V tile
     constexpr int CH = D / 16;                   // 16-byte chunks per row
@@ -43,8 +43,9 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
     constexpr int OFF_KS = 0;                            // two fp32 k_scale vectors
     constexpr int OFF_XM = 2 * BN * 4;                   // 4 waves x 32 rows fp32: partial row maxima / row sums
     constexpr int OFF_XP = OFF_XM + 4 * 32 * 4;          // 4 waves x 64 lanes x 16 bytes: the waves' P8 fragments
-    constexpr int OFF_VS = OFF_XP + 4 * 64 * 16;         // VBLK: two vectors of D fp32 channel scales
-    constexpr int OFF_K = OFF_VS + (VBLK ? 2 * D * 4 : 0);
+    constexpr int OFF_VS = OFF_XP + 4 * 64 * 16;         // VBLK: two vectors of NBS * D fp32 channel scales (one row per block)
+    constexpr int NV = NBS * D;                          // channel scales per step
+    constexpr int OFF_K = OFF_VS + (VBLK ? 2 * NV * 4 : 0);
     constexpr int OFF_V = OFF_K + 2 * KT;
     constexpr int LDS_BYTES = OFF_V + 2 * VT;
     static_assert(OFF_K % 256 == 0, "tiles keep the bank alignment the swizzles assume");
@@ -109,15 +110,22 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
     const KScaleSource ks_src(p, b, hk, seqlen_k);
     auto load_ks = [&](int nb) __attribute__((always_inline)) -> uint32_t { return ks_src.load(nb * BNB + (tid & (BN - 1))); };
     auto cvt_ks = [&](uint32_t raw) __attribute__((always_inline)) -> float { return ks_src.cvt(raw); };
-    // VBLK: fp32 channel scales of a key block; thread 128 + c fetches channel c
-    const int vs_c = tid - 128;
+    // VBLK: fp32 channel scales of the step's key blocks, NV = NBS * D values.  Up to 128 values: thread 128 + i fetches
+    // value i (block i / D, channel i % D); 512 values (head_dim 256): thread t fetches channel t of both blocks.
     // (per-wave tests, scalar branches: see fwd_full_int8_kernel)
+    constexpr int VPT = NV > 128 ? NV / kThreads : 1;         // values per fetching thread
     const bool ks_wave = wave < BN / 64;
-    const bool vs_thread = VBLK && wave >= 2 && (wave - 2) * 64 < D;
-    const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + (vs_thread ? vs_c : 0));
-    auto load_vs = [&](int nb) __attribute__((always_inline)) -> float {
+    const bool vs_thread = VBLK && (NV > 128 || (wave >= 2 && (wave - 2) * 64 < NV));
+    const int vs_i = NV > 128 ? tid : (vs_thread ? tid - 128 : 0);
+    const int vs_blk0 = NV > 128 ? 0 : vs_i / D;              // block (inside the step) of the thread's first value
+    const float* Vsg = (const float*)p.v_scale + (b * p.vs_sb + hk * p.vs_sh + vs_i % D);
+    const int vs_last_row = VBLK ? ((p.seqlen_k + BNB - 1) / BNB - 1) / p.vs_g : 0;
+    // (a step's second block may lie past the end of the sequence: its keys are hidden, any scale row serves)
+    auto load_vs = [&](int nb, int j) __attribute__((always_inline)) -> float {
         if (!VBLK) return 0.f;
-        const int row = p.vs_g == 1 ? nb : nb / p.vs_g;       // (VBLK: one block per step)
+        const int blk = nb + vs_blk0 + j;
+        int row = p.vs_g == 1 ? blk : blk / p.vs_g;
+        row = row < vs_last_row ? row : vs_last_row;
         return Vsg[(int64_t)row * p.vs_sblk];
     };
 
@@ -144,8 +152,8 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
     const uint32_t xm_rd = OFF_XM + 4 * lq;                          // + 128 per wave
     const uint32_t xp_wr = OFF_XP + 1024 * wave + 16 * lane;
     const uint32_t xp_rd = OFF_XP + 16 * lane;                       // + 1024 per wave
-    const uint32_t vs_wr = OFF_VS + 4 * (vs_thread ? vs_c : 0);
-    const uint32_t vs_rd = OFF_VS + 16 * lh;                         // + 4 * (32*dt + 8*a4) per read
+    const uint32_t vs_wr = OFF_VS + 4 * vs_i;                        // + 4 * kThreads per further value
+    const uint32_t vs_rd = OFF_VS + 16 * lh;                         // + 4 * (D*blk + 32*dt + 8*a4) per read
     // head_dim 64 has two output tiles for four waves: waves 2 and 3 compute tiles 0 and 1 a second time and store
     // nothing (the same instruction stream for every wave; a run-time "owns a tile" test around the V fragments and the
     // accumulator update costs the owners a hundred register copies per step)
@@ -156,16 +164,19 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
 
     auto step = [&](auto buf_tag, int nb) __attribute__((always_inline)) {
         constexpr int BUF = decltype(buf_tag)::value ? 1 : 0;
-        constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4, VSB = BUF * D * 4;
+        constexpr int KB = BUF * KT, VB = BUF * VT, SB = BUF * BN * 4, VSB = BUF * NV * 4;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();                                   // tile nb has landed; the other buffer and the exchange areas are free
         const bool more = nb + NBS < nb_end;
         uint32_t ks_next = 0;
-        float vs_next = 0.f;
+        float vs_next[VPT] = {};
         if (more) {
             issue_loads(nb + NBS, BUF ^ 1);
             if (ks_wave) ks_next = load_ks(nb + NBS);
-            if (vs_thread) vs_next = load_vs(nb + NBS);
+            if (vs_thread) {
+#pragma unroll
+                for (int j = 0; j < VPT; ++j) vs_next[j] = load_vs(nb + NBS, j);
+            }
         }
         // -------- S^T of this wave's 32 keys, dequantise, partial row maximum
         v4i fr[KS];
@@ -244,13 +255,15 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
             }
         }
         *(v4i*)(smem + xp_wr) = p8;
-        v4f vsc[DTW][4];
+        v4f vsc[NBS][DTW][4];                              // channel scales of the step's blocks for this wave's output tiles
         if (VBLK) {
 #pragma unroll
-            for (int j = 0; j < DTW; ++j)
+            for (int blk = 0; blk < NBS; ++blk)
 #pragma unroll
-                for (int a4 = 0; a4 < 4; ++a4)
-                    vsc[j][a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (32 * ((wave + 4 * j) % DT) + 8 * a4));
+                for (int j = 0; j < DTW; ++j)
+#pragma unroll
+                    for (int a4 = 0; a4 < 4; ++a4)
+                        vsc[blk][j][a4] = *(const v4f*)(smem + vs_rd + VSB + 4 * (D * blk + 32 * ((wave + 4 * j) % DT) + 8 * a4));
         }
         __syncthreads();                                   // the four P8 fragments are in LDS
         v4i pall[NST];
@@ -265,7 +278,7 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
                 for (int st = 0; st < NST; ++st) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[j][st], pall[st], acc, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    if (VBLK) o_acc[j][r] = fmaf(o_acc[j][r], alpha, (float)acc[r] * vsc[j][r >> 2][r & 3]);
+                    if (VBLK) o_acc[j][r] = fmaf(o_acc[j][r], alpha, (float)acc[r] * vsc[0][j][r >> 2][r & 3]);
                     else o_acc[j][r] = fmaf(o_acc[j][r], alpha, (float)acc[r]);
                 }
             } else {
@@ -275,7 +288,11 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
 #pragma unroll
                 for (int st = NST / 2; st < NST; ++st) acc_b = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[j][st], pall[st], acc_b, 0, 0, 0);
 #pragma unroll
-                for (int r = 0; r < 16; ++r) o_acc[j][r] = fmaf(fmaf(o_acc[j][r], alpha, (float)acc_a[r]), alpha_b, (float)acc_b[r]);
+                for (int r = 0; r < 16; ++r) {
+                    if (VBLK) o_acc[j][r] = fmaf(fmaf(o_acc[j][r], alpha, (float)acc_a[r] * vsc[0][j][r >> 2][r & 3]), alpha_b,
+                                                 (float)acc_b[r] * vsc[NBS - 1][j][r >> 2][r & 3]);
+                    else o_acc[j][r] = fmaf(fmaf(o_acc[j][r], alpha, (float)acc_a[r]), alpha_b, (float)acc_b[r]);
+                }
             }
         }
         if (NBS == 1) l_run = fmaf(l_run, alpha, lsum);
@@ -284,13 +301,19 @@ __global__ void __launch_bounds__(kThreads, D <= 128 ? 2 : 1) fwd_decode_full_in
         // for the next step's tile copies that were issued ahead of it - that wait belongs at the end of the step)
         asm volatile("" : "+v"(ks_next));
         if (more && ks_wave) *(float*)(smem + ks_wr + (BUF ^ 1) * BN * 4) = cvt_ks(ks_next);
-        if (more && vs_thread) *(float*)(smem + vs_wr + (BUF ^ 1) * D * 4) = vs_next;
+        if (more && vs_thread) {
+#pragma unroll
+            for (int j = 0; j < VPT; ++j) *(float*)(smem + vs_wr + (BUF ^ 1) * NV * 4 + j * kThreads * 4) = vs_next[j];
+        }
     };
 
     if (nb_begin < nb_end) {
         issue_loads(nb_begin, 0);
         if (ks_wave) *(float*)(smem + ks_wr) = cvt_ks(load_ks(nb_begin));
-        if (vs_thread) *(float*)(smem + vs_wr) = load_vs(nb_begin);
+        if (vs_thread) {
+#pragma unroll
+            for (int j = 0; j < VPT; ++j) *(float*)(smem + vs_wr + j * kThreads * 4) = load_vs(nb_begin, j);
+        }
         int nb = nb_begin;
         while (true) {
             if (nb >= nb_end) break;

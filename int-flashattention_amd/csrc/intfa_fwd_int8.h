@@ -14,14 +14,20 @@
 #pragma once
 #include "intfa_device.h"
 
+#ifndef INTFA_D64_WAVES
+#define INTFA_D64_WAVES 0
+#endif
+
 namespace intfa {
 
 // Key block length of the full-int8 kernels: 128 keys, or 64 at head_dim 256 (registers and LDS).  At head_dim 256 this
 // kernel only serves the int32 S export; the forward itself is fwd_full_int8_pair_kernel (intfa_fwd_int8_pair.h), which
 // spreads the 256 output columns of a query row over two waves.
 template <int D> struct FullInt8Geom {
-    static constexpr int NST = D <= 128 ? 4 : 2;
+    static constexpr int NST = D == 128 ? 4 : 2;
     static constexpr int BN = 32 * NST;
+    // occupancy the register budget is held to (a workgroup puts one wave on each SIMD: workgroups per compute unit)
+    static constexpr int waves_per_simd(bool causal, int vblk) { return D == 64 ? (INTFA_D64_WAVES ? INTFA_D64_WAVES : (causal || vblk ? 3 : 4)) : 2; }
 };
 
 // VBLK != 0: V carries one scale per key block and channel (layout of the reference's CUDA kernel,
@@ -32,7 +38,7 @@ template <int D> struct FullInt8Geom {
 // 128-key block (the running maximum and P8 are those of intfa_fwd_block_n()), but P V is summed in int32 per 64-key
 // half and each half is multiplied by its own scale row.
 template <int D, bool CAUSAL, int OUT_DT /*0 f16, 1 bf16*/, int PROUND, bool DUMP_S, bool SPLIT, int VBLK = 0>
-__global__ void __launch_bounds__(kThreads, 2) fwd_full_int8_kernel(const KParams p) {
+__global__ void __launch_bounds__(kThreads, FullInt8Geom<D>::waves_per_simd(CAUSAL, VBLK)) fwd_full_int8_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the kernel's symbol
     constexpr int KS = D / 32;                   // k-steps of Q K^T (32 bytes of head_dim each)
     static_assert(D <= 128 || DUMP_S, "head_dim 256 runs fwd_full_int8_pair_kernel");

@@ -55,8 +55,7 @@ INTFA_DECL_LAUNCH(launch_full_int8_d256);
 INTFA_DECL_LAUNCH(launch_full_int8_vblk_d64);     // per-block, per-channel V scales
 INTFA_DECL_LAUNCH(launch_full_int8_vblk_d128);
 INTFA_DECL_LAUNCH(launch_full_int8_vblk_d256);
-INTFA_DECL_LAUNCH(launch_full_int8_vblk64_d64);   // V scale rows of 64 keys (two per key block)
-INTFA_DECL_LAUNCH(launch_full_int8_vblk64_d128);
+INTFA_DECL_LAUNCH(launch_full_int8_vblk64_d128);  // V scale rows of 64 keys (two per 128-key block)
 INTFA_DECL_LAUNCH(launch_decode_full_int8_d64);    // few query rows per head: the waves of a workgroup share the keys
 INTFA_DECL_LAUNCH(launch_decode_full_int8_d128);
 INTFA_DECL_LAUNCH(launch_decode_full_int8_d256);

@@ -15,7 +15,9 @@ import intfa_oracle as O  # noqa: E402
 
 
 def main():
-    B, H, N, D = 1, 1, 160, 64                      # N is not a multiple of 128 on purpose
+    B, H, N, D = 1, 1, 160, 64                      # N is not a multiple of the 128-row query block on purpose
+    # (the full-int8 kernel's key block at head_dim 64 is 64: the reference admits none longer than head_dim,
+    # flash_atten_full_int8.py:88)
     q, k, v, _ = O.make_inputs(B, H, N, D, seed=2024)
     q8, qs = O.quant_pertoken(q)
     k8, ks = O.quant_pertoken(k)
@@ -26,8 +28,8 @@ def main():
                s_int32=O.qk_int32(q8, k8).numpy())
     for causal in (False, True):
         tag = "causal" if causal else "dense"
-        out[f"full_ref_{tag}"] = O.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, block_n=128).numpy()
-        out[f"full_rne_{tag}"] = O.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, block_n=128, p_requant=O.p_requant_rne).numpy()
+        out[f"full_ref_{tag}"] = O.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, block_n=64).numpy()
+        out[f"full_rne_{tag}"] = O.attention_full_int8(q8, k8, v8, qs, ks, vs, causal, sm, block_n=64, p_requant=O.p_requant_rne).numpy()
         out[f"half_{tag}"] = O.attention_int8(q8, k8, v, qs, ks, causal, sm, block_n=64).numpy()
         out[f"fp_{tag}"] = O.attention_fp(q, k, v, causal, sm, block_n=64).numpy()
     np.savez_compressed(os.path.join(os.path.dirname(os.path.abspath(__file__)), "attention_small.npz"), **out)

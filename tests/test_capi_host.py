@@ -28,6 +28,7 @@ def test_library_exports_every_declared_symbol():
     header_version = int(re.search(r"#define INTFA_VERSION (\d+)", text).group(1))
     assert lib.intfa_version() == header_version == _capi.ABI_VERSION
     assert lib.intfa_fwd_block_n(0, 128) == 128 == _host.BLOCK
+    assert lib.intfa_fwd_block_n(0, 64) == 64      # never longer than head_dim (flash_atten_full_int8.py:88)
     assert lib.intfa_fwd_block_n(0, 256) == 64 and lib.intfa_fwd_block_n(1, 128) == 64 and lib.intfa_fwd_block_n(2, 64) == 64
     assert lib.intfa_fwd_block_n(3, 128) < 0 and lib.intfa_fwd_block_n(0, 96) < 0
 

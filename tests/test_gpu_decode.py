@@ -202,7 +202,7 @@ def test_causal_decode_matches_oracle(B, H, H_kv, Nq, Nk, D, p_round):
     rep = lambda t: t.repeat_interleave(x["g"], dim=1)
     rq = O.p_requant_rne if p_round == "rne" else O.p_requant_reference
     ref, lse_ref = O.attention_full_int8(x["q8"], rep(x["k8"]), rep(x["v8"]), x["qs"], rep(x["ks"]), rep(x["vs"]), True, sm,
-                                         block_n=128, p_requant=rq, return_lse=True)
+                                         block_n=M.block_n("full", D), p_requant=rq, return_lse=True)
     assert torch.isfinite(o).all()
     empty = max(Nq - Nk, 0)
     if empty:

@@ -112,7 +112,7 @@ def identity_v(B, H, Nk, D, shift):
     return v8
 
 
-@pytest.mark.parametrize("D,Nq,Nk", [(128, 128, 128), (128, 384, 128), (64, 256, 128), (256, 128, 64), (128, 16, 128), (64, 33, 128)])
+@pytest.mark.parametrize("D,Nq,Nk", [(128, 128, 128), (128, 384, 128), (64, 256, 64), (256, 128, 64), (128, 16, 128), (64, 33, 64)])
 @pytest.mark.parametrize("pattern", ["powers_of_two", "random"])
 def test_reference_rounding_packs_every_byte(D, Nq, Nk, pattern):
     """One key block, V = identity (shifted to reach the keys beyond head_dim): P8 read back from the output."""

@@ -60,10 +60,10 @@ def test_quant_perblock_channel_strided_input():
     # 64-key scale rows under the 128-key block: the granularity of the reference's CUDA kernel (kBlockN = 64 at
     # head_dim 128, csrc/flash_fwd_launch_template.h:514-519); P V is summed per 64-key half
     (1, 2, 512, 128, False, 0.5),
-    (2, 2, 384, 64, True, 0.5),
+    (2, 2, 384, 64, True, 2),          # head_dim 64: 64-key blocks, one scale row per two of them
     (1, 3, 300, 128, True, 0.5),       # ragged: the last block holds 44 keys, its second scale row does not exist
     (1, 2, 200, 128, False, 0.5),      # the last block's second half holds 8 keys
-    (1, 2, 160, 64, False, 0.5),
+    (1, 2, 160, 64, False, 1),         # head_dim 64: a scale row per 64-key block is the kernel's own block
     (1, 2, 40, 128, True, 0.5),        # few query rows (the decode-shaped kernel has no 64-key rows: the general one runs)
 ])
 @pytest.mark.parametrize("p_round", ["rne", "reference"])
@@ -163,15 +163,15 @@ def test_64_key_v_scale_rows_with_grouped_heads_split_kv_decode_shapes_and_bf16(
 def test_blocked_v_scale_small_head_dim_and_argument_checks():
     x = blocked_inputs(1, 2, 256, 32, 84, 128)
     o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, 0.2, v_scale_block=128, p_round="rne")
-    ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], False, 0.2, block_n=128,
+    ref = O.attention_full_int8(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"], False, 0.2, block_n=64,
                                 v_scale_block=128, p_requant=O.p_requant_rne)
     assert_same_rounding(o, ref)
-    with pytest.raises(RuntimeError):                          # 32 neither is a multiple of the 128-key block nor 64
+    with pytest.raises(RuntimeError):                          # 32 is not a multiple of the 64-key block
         v8, vs = O.quant_perblock_channel(x["v"], 32)
         M.attention_full_int8(*gpu(x["q8"], x["k8"], v8, x["qs"], x["ks"], vs), False, 0.2, v_scale_block=32, p_round="rne")
-    with pytest.raises(RuntimeError):                          # 192 is a multiple of 64 only
-        v8, vs = O.quant_perblock_channel(x["v"], 192)
-        M.attention_full_int8(*gpu(x["q8"], x["k8"], v8, x["qs"], x["ks"], vs), False, 0.2, v_scale_block=192, p_round="rne")
+    with pytest.raises(RuntimeError):                          # neither is 96
+        v8, vs = O.quant_perblock_channel(x["v"], 96)
+        M.attention_full_int8(*gpu(x["q8"], x["k8"], v8, x["qs"], x["ks"], vs), False, 0.2, v_scale_block=96, p_round="rne")
     with pytest.raises(ValueError):                            # wrong number of scale rows
         M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"][:, :, :1]), False, 0.2, v_scale_block=128, p_round="rne")
     with pytest.raises(ValueError):

@@ -72,7 +72,7 @@ def test_static_scratch_entry_point_equals_the_workspace_entry_point_on_two_call
         assert torch.equal(o_st, o_ws) and torch.equal(lse_st, lse_ws)
         # and both are the oracle's split evaluation (reference rounding) where the oracle has one (equal lengths or not causal)
         if not pb["causal"]:
-            ref = O.attention_full_int8_splitkv(*pb["cpu"], False, pb["D"] ** -0.5, splits, block_n=128)
+            ref = O.attention_full_int8_splitkv(*pb["cpu"], False, pb["D"] ** -0.5, splits, block_n=64 if pb["D"] != 128 else 128)
             assert (o_st.float().cpu() - ref.float()).abs().max().item() <= 2e-2
     # a single pass needs no scratch at all and is the plain entry point
     (o_ws, lse_ws), (o_st, lse_st) = run_both(small, 1)
