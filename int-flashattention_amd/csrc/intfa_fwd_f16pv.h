@@ -3,8 +3,9 @@
 //
 // Same tiling as the full-int8 kernel (4 waves x 32 query rows, S^T = K Q^T so that a lane owns one query
 // column), but keys go in blocks of 64 (two 32-key sub-tiles) and P is cast to V's 16-bit type in registers
-// and multiplied on v_mfma_f32_32x32x16_{f16,bf16}, whose fp32 accumulator IS the running output: per block the
-// accumulator is scaled by alpha and the MFMA adds P V on top (acc = tl.dot(p, v, acc), flash_atten_int8.py:59).
+// and multiplied on v_mfma_f32_32x32x16_{f16,bf16}, whose fp32 accumulator IS the running output: the MFMA adds P V on
+// top (acc = tl.dot(p, v, acc), flash_atten_int8.py:59); the rescaling by alpha of flash_atten_int8.py:48-52 happens only
+// in the blocks where a row's maximum rises by more than kFrameSlack over the exponent's reference point (see below).
 // V rows stay row-major in LDS; the transposing 8-byte load (ds_read_b64_tr_b16) delivers the A operand.
 #pragma once
 #include "intfa_device.h"
@@ -13,6 +14,7 @@
 namespace intfa {
 
 constexpr int kBlockN16 = 64;      // key block of this kernel
+constexpr float kFrameSlack = 8.f; // how far a row's block maximum may exceed the exponent's frame before the frame moves
 
 __device__ __forceinline__ v8h pack_p_f16(const float* e) {
     v8h r;
@@ -237,9 +239,24 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
         load_vfrags(vf[0], 0);
         if (1 < DT) load_vfrags(vf[1], 1);
         mx = half_pair_max(mx);
-        const float m_new = fmaxf(m_run, mx * qsc);
-        const float alpha = fast_exp2(m_run - m_new);
-        m_run = m_new;
+        // The exponent's reference point ("frame") follows the running maximum lazily: it moves, and the output and the row
+        // sum are rescaled as the reference does in every block (flash_atten_int8.py:48-52), only when some row's block
+        // maximum exceeds its frame by more than kFrameSlack.  P is a 16-bit FLOATING-point number here: p' = exp2(x - frame)
+        // <= 2^kFrameSlack differs from the reference's p = exp2(x - m_new) by a factor that is the same for the numerator
+        // sum p' v and for the row sum, so acc / l and m + log2(l) are unchanged; only the 16-bit rounding of the single
+        // p' lands on other values (relative 2^-12, unbiased).  In the common case no vector instruction touches the output.
+        const float mxs = mx * qsc;
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(mxs > m_run + kFrameSlack) != 0, 0)) {
+            const float m_mv = fmaxf(m_run, mxs);
+            const float a_mv = fast_exp2(m_run - m_mv);
+            m_run = m_mv;
+            l_run *= a_mv;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o_acc[dt][r] *= a_mv;
+        }
+        const float m_new = m_run;
         // -------- pass 2: P = exp2(x*qsc - m), row sum, cast to the 16-bit type
         float lsum = 0.f;
         v4i pf[NST][2];                                   // B operands: 8 x 16-bit per 16-key step
@@ -255,12 +272,9 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
                 pf[st][u] = IO_DT == 0 ? __builtin_bit_cast(v4i, pack_p_f16(e + 8 * u)) : __builtin_bit_cast(v4i, pack_p_bf16(e + 8 * u));
             asm volatile("" : "+v"(lsum));
         }
-        l_run = fmaf(l_run, alpha, lsum);
-        // -------- O^T[d, q] = alpha * O^T + V^T[d, key] P^T[key, q]: d-tile 0 is rescaled here, d-tile dt+1 under the
-        // MFMAs of d-tile dt
+        l_run += lsum;
+        // -------- O^T[d, q] += V^T[d, key] P^T[key, q] (the fp32 accumulators of the MFMAs are the running output)
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { o_acc[0][r] *= alpha; asm volatile("" : "+v"(o_acc[0][r])); }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
@@ -269,13 +283,6 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
                 __builtin_amdgcn_sched_barrier(0);
                 if (!(DIAG && st > gw)) o_acc[dt] = mfma16(vf[dt & 1][st][u], pf[st][u], o_acc[dt]);
                 __builtin_amdgcn_sched_barrier(0);
-                if (dt + 1 < DT) {
-#pragma unroll
-                    for (int b4 = 0; b4 < 4; ++b4) {
-                        o_acc[dt + 1][4 * a4 + b4] *= alpha;
-                        asm volatile("" : "+v"(o_acc[dt + 1][4 * a4 + b4]));
-                    }
-                }
             }
             __builtin_amdgcn_sched_barrier(0);
             if (dt + 2 < DT) load_vfrags(vf[dt & 1], dt + 2);

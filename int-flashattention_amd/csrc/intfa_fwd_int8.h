@@ -14,10 +14,6 @@
 #pragma once
 #include "intfa_device.h"
 
-#ifndef INTFA_D64_WAVES
-#define INTFA_D64_WAVES 0
-#endif
-
 namespace intfa {
 
 // Key block length of the full-int8 kernels: 128 keys, or 64 at head_dim 256 (registers and LDS).  At head_dim 256 this
@@ -27,7 +23,7 @@ template <int D> struct FullInt8Geom {
     static constexpr int NST = D == 128 ? 4 : 2;
     static constexpr int BN = 32 * NST;
     // occupancy the register budget is held to (a workgroup puts one wave on each SIMD: workgroups per compute unit)
-    static constexpr int waves_per_simd(bool causal, int vblk) { return D == 64 ? (INTFA_D64_WAVES ? INTFA_D64_WAVES : (causal || vblk ? 3 : 4)) : 2; }
+    static constexpr int waves_per_simd(bool causal, int vblk) { return D == 64 ? (causal || vblk ? 3 : 4) : 2; }
 };
 
 // VBLK != 0: V carries one scale per key block and channel (layout of the reference's CUDA kernel,

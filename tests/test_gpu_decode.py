@@ -359,13 +359,46 @@ def test_decode_head_dim_256_per_batch_key_lengths(causal):
         assert torch.equal(o[b:b + 1], ob) and torch.equal(lse[b:b + 1], lb), f"batch entry {b} (length {n})"
 
 
-def test_decode_head_dim_256_blocked_v_scales_stay_with_the_general_kernel():
-    """Few rows, head_dim 256, per-block per-channel V scales: the call is not a shape of the decode kernel (it has one V
-    scale per (batch, head) at this head_dim) and still comes out right."""
-    B, H, Nq, Nk, D = 1, 2, 4, 600, 256
-    x = decode_inputs(B, H, H, Nq, Nk, D, seed=114, v_block=128)
+@pytest.mark.parametrize("B,H,H_kv,Nq,Nk,D,vsb,causal,splits", [
+    (1, 2, 2, 4, 600, 256, 128, False, 1),      # one scale row per two 64-key blocks: both blocks of a step share it
+    (2, 4, 4, 1, 1000, 256, 64, False, 1),      # one scale row per block: blocks A and B of a step have their own
+    (1, 8, 2, 3, 333, 256, 64, True, 1),        # grouped heads folded into rows, causal (causal_rows), ragged last step
+    (1, 2, 2, 33, 577, 256, 64, True, 3),       # two 32-row workgroups, split-KV over whole-sequence ranges
+    (2, 2, 1, 5, 777, 64, 64, False, 1),        # head_dim 64: two 64-key blocks per step as well
+    (1, 4, 2, 8, 450, 64, 128, True, 2),
+    (1, 2, 2, 64, 64, 64, 64, True, 1),         # a single block: the step's second block does not exist
+])
+@pytest.mark.parametrize("p_round", ["reference", "rne"])
+def test_decode_with_blocked_v_scales_and_two_blocks_per_step(B, H, H_kv, Nq, Nk, D, vsb, causal, splits, p_round):
+    """Few query rows with per-block, per-channel V scales at the head dims whose decode step covers two 64-key blocks
+    (64 and 256): each block's int32 P V is multiplied by its own scale row (csrc/mask.h:313-340), as in the general kernel."""
+    bn = M.block_n("full", D)
+    assert bn == 64
+    x = decode_inputs(B, H, H_kv, Nq, Nk, D, seed=114 + D + vsb, v_block=vsb)
     sm = D ** -0.5
-    o = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), False, sm, v_scale_block=128, p_round="rne")
+    o, lse = M.attention_full_int8(*gpu(x["q8"], x["k8"], x["v8"], x["qs"], x["ks"], x["vs"]), causal, sm, v_scale_block=vsb,
+                                   p_round=p_round, num_splits=splits, return_lse=True)
     torch.cuda.synchronize()
-    ref = oracle(x, sm, 64, p_requant=O.p_requant_rne, v_scale_block=128)
-    assert max_abs(o, ref) <= 4e-3 and mean_rel(o, ref) <= 1e-3
+    rq = O.p_requant_rne if p_round == "rne" else O.p_requant_reference
+    rep = lambda t: t.repeat_interleave(x["g"], dim=1)
+    a = (x["q8"], rep(x["k8"]), rep(x["v8"]), x["qs"], rep(x["ks"]), rep(x["vs"]))
+    if splits == 1:
+        ref, lse_ref = O.attention_full_int8(*a, causal, sm, block_n=bn, p_requant=rq, v_scale_block=vsb, return_lse=True)
+        assert_same_rounding(o, ref)
+        assert (lse.cpu() - lse_ref).abs().max().item() <= 1e-3
+    else:
+        # decode-shaped calls deal the blocks of the whole sequence to the splits, masked or not
+        nblk = (Nk + bn - 1) // bn
+        per = (nblk + splits - 1) // splits
+        o_parts = torch.zeros((splits, B, H, Nq, D)); lse_parts = torch.full((splits, B, H, Nq), float("-inf"))
+        for s_ in range(splits):
+            b0, b1 = s_ * per, min((s_ + 1) * per, nblk)
+            if b0 >= b1:
+                continue
+            acc, l, m = O._blocked_forward("full", *a, causal, sm, 128, bn, key_lo=b0 * bn, key_hi=min(b1 * bn, Nk), p_requant=rq,
+                                           v_scale_block=vsb)
+            seen = ~torch.isinf(m)
+            o_parts[s_] = torch.where(seen[..., None], acc / l[..., None], torch.zeros_like(acc))
+            lse_parts[s_] = torch.where(seen, m + torch.log2(l), torch.full_like(m, float("-inf")))
+        ref, _ = O.splitkv_combine(o_parts, lse_parts)
+        assert max_abs(o, ref.half()) <= 2e-3 and mean_rel(o, ref.half()) <= 2e-4

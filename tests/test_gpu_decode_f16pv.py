@@ -114,16 +114,19 @@ def test_decode_matches_oracle(B, H, H_kv, Nq, Nk, D, causal, variant, dtype):
 @pytest.mark.parametrize("D", [64, 128, 256])
 @pytest.mark.parametrize("causal", [False, True])
 def test_decode_kernel_agrees_with_the_general_kernel(variant, D, causal):
-    """65 query rows run the general kernel, 64 of them alone the decode kernel: same block maxima, same 16-bit P and the
-    same MFMA steps per block, so a row's result differs only through the order of the fp32 row-sum additions (one
-    rounding of the 16-bit output now and then).  With the mask the 64 rows are the LAST 64 of the 65 (the mask is aligned
-    to the end of the cache)."""
+    """65 query rows run the general kernel, 64 of them alone the decode kernel.  At head_dim 256 both take the same block
+    maxima, the same 16-bit P and the same MFMA steps per block, so a row's result differs only through the order of the
+    fp32 row-sum additions (one rounding of the 16-bit output now and then).  At head_dim <= 128 the general kernel takes
+    exp2 against a reference point that lags the running maximum (it rescales the output only when a row's maximum rises by
+    more than 8), the decode kernel against the running maximum itself as the oracle does: the same p up to a factor that
+    cancels in acc / l, rounded to 16 bits at another place (relative 2^-12 per element, unbiased) - a few 1e-4 in the mean.
+    With the mask the 64 rows are the LAST 64 of the 65 (the mask is aligned to the end of the cache)."""
     q, k, v = inputs(1, 2, 2, 65, 1500, D, seed=3100 + D)
     sm = D ** -0.5
     general, lg = run(variant, q, k, v, causal, sm, return_lse=True)
     rows = slice(1, 65) if causal else slice(0, 64)
     decode, ld = run(variant, q[:, :, rows].contiguous(), k, v, causal, sm, return_lse=True)
-    assert max_abs(decode, general[:, :, rows]) <= 1e-3 and mean_rel(decode, general[:, :, rows]) <= 2e-5
+    assert max_abs(decode, general[:, :, rows]) <= 1e-3 and mean_rel(decode, general[:, :, rows]) <= (2e-5 if D == 256 else 6e-4)
     assert (ld - lg[:, :, rows]).abs().max().item() <= 1e-4
 
 

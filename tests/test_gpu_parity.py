@@ -734,7 +734,13 @@ def test_other_benchmark_shapes_one_slice_against_oracle(variant, B, H, N, D, ca
             ref = O.attention_full_int8(cpu(q8), cpu(k8), cpu(v8), cpu(qs), cpu(ks), cpu(vs), causal, sm, block_n=bn,
                                         p_requant=O.p_requant_rne)
     assert torch.isfinite(o).all()
-    assert max_abs(o[b:b + 1, h:h + 1], ref) <= 4e-3 and mean_rel(o[b:b + 1, h:h + 1], ref) <= 2e-4
+    # full-int8: the kernel and the oracle quantise the same P8 (only exp2 differs in the last place).  The 16-bit-P kernels
+    # at head_dim <= 128 take exp2 against a reference point that lags the running maximum (the output is rescaled only
+    # when a row's maximum rises by more than 8): the same p times a power-of-two-free factor, so its 16-bit rounding lands
+    # elsewhere than the oracle's (relative 2^-12 per element, unbiased) - a few 1e-4 in the mean on outputs that are sums
+    # of thousands of products with random signs, far inside the 1e-2 of the stated tolerance.
+    tol_rel = 2e-4 if variant == "full" or D == 256 else 6e-4
+    assert max_abs(o[b:b + 1, h:h + 1], ref) <= 4e-3 and mean_rel(o[b:b + 1, h:h + 1], ref) <= tol_rel
 
 
 # ------------------------------------------------------------------------------------------ HIP graph capture
