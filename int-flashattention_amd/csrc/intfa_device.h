@@ -74,7 +74,8 @@ struct KParams {
     // workgroup -> work mapping of this launch (set by finish_mapping() in intfa_launch.h from the grid size)
     int32_t per_head;                      // workgroups per query head
     int32_t heads_kv;                      // heads / kv_group
-    int32_t xcd_deal;                      // 1: the K/V heads divide evenly among the 8 XCDs
+    int32_t xcd_whole_wgs;                 // workgroups of the K/V heads that are dealt whole to the 8 XCDs (a multiple of 8)
+    int32_t xcd_rem_chunk;                 // the remaining heads: consecutive workgroups per XCD (0: dealt one by one)
     FastDiv d_per_kv, d_heads_kv, d_per_head, d_n_split, d_heads, d_kv_group;
 };
 
@@ -99,6 +100,9 @@ __device__ __forceinline__ float load_scale(const char* base, int64_t idx, int d
 // the 8 XCDs, each with its own L2: every XCD gets whole K/V heads, so the K/V tiles of a head are re-read from one L2.
 // With grouped K/V heads (kv_group query heads share one K/V head) the unit dealt to an XCD is the K/V head: all query
 // heads of a group run on the XCD whose L2 holds their K/V.
+// When the number of (batch, K/V head) pairs is no multiple of 8, the first 8 * floor(pairs / 8) are dealt whole as above and
+// the workgroups of the remaining pairs, taken in head order, are cut into 8 equal runs, one per XCD: a remaining head's
+// K/V then reaches two or three L2s instead of all eight.
 // (All divisors are fixed per launch: fast_div.)
 struct WorkgroupJob { int b, h, hk, rem; };      // batch entry, query head, K/V head, index among the head's workgroups
 __device__ __forceinline__ WorkgroupJob deal_workgroup(const KParams& p, int bid) {
@@ -106,14 +110,17 @@ __device__ __forceinline__ WorkgroupJob deal_workgroup(const KParams& p, int bid
     const int per_head = p.per_head;
     const int per_kv = per_head * kv_group;              // workgroups per K/V head
     int kv_lin, r;
-    if (p.xcd_deal) {
+    if (bid < p.xcd_whole_wgs) {
         const int xcd = bid & 7, slot = bid >> 3;
         const int q = fast_div(slot, p.d_per_kv);
         kv_lin = q * 8 + xcd;
         r = slot - q * per_kv;
     } else {
-        kv_lin = fast_div(bid, p.d_per_kv);
-        r = bid - kv_lin * per_kv;
+        const int j = bid - p.xcd_whole_wgs;                        // (xcd_whole_wgs is a multiple of 8: j & 7 is the XCD)
+        const int idx = p.xcd_rem_chunk ? (j & 7) * p.xcd_rem_chunk + (j >> 3) : j;
+        const int q = fast_div(idx, p.d_per_kv);
+        kv_lin = fast_div(p.xcd_whole_wgs, p.d_per_kv) + q;
+        r = idx - q * per_kv;
     }
     const int bb = fast_div(kv_lin, p.d_heads_kv), hk = kv_lin - bb * p.heads_kv;
     const int hq = fast_div(r, p.d_per_head);            // query head inside the group

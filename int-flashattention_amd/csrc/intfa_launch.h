@@ -29,7 +29,9 @@ inline KParams finish_mapping(const KParams& kp, int grid) {
     const int n_split = kp.num_splits > 1 ? kp.num_splits : 1;
     k.per_head = grid / (kp.batch * kp.heads);
     k.heads_kv = kp.heads / kp.kv_group;
-    k.xcd_deal = ((kp.batch * k.heads_kv) & 7) == 0 ? 1 : 0;
+    const int per_kv = k.per_head * kp.kv_group, units = kp.batch * k.heads_kv;
+    k.xcd_whole_wgs = (units / 8) * 8 * per_kv;
+    k.xcd_rem_chunk = ((units % 8) * per_kv) % 8 == 0 ? (units % 8) * per_kv / 8 : 0;
     k.d_per_kv = make_fast_div(k.per_head * kp.kv_group);
     k.d_heads_kv = make_fast_div(k.heads_kv);
     k.d_per_head = make_fast_div(k.per_head);

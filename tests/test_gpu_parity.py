@@ -689,6 +689,66 @@ def test_headline_shape_slices_reproduce_and_v_scale_is_linear():
     ref = O.attention_full_int8(cpu(q8), cpu(k8), cpu(v8), cpu(qs), cpu(ks), cpu(vs), False, sm, block_n=128,
                                 p_requant=O.p_requant_rne)
     assert max_abs(o[b:b + 1, h:h + 1], ref) <= 2e-3 and mean_rel(o[b:b + 1, h:h + 1], ref) <= 2e-4
+    # the default (the reference's rounding of P) at the same size: same-rounding agreement with the oracle, and the
+    # opt-in rounding stays inside the stated tolerance of the reference's result
+    o_ref = M.attention_full_int8(q8, k8, v8, qs, ks, vs, False, sm)
+    ref_r = O.attention_full_int8(cpu(q8), cpu(k8), cpu(v8), cpu(qs), cpu(ks), cpu(vs), False, sm, block_n=128)
+    assert max_abs(o_ref[b:b + 1, h:h + 1], ref_r) <= 2e-3 and mean_rel(o_ref[b:b + 1, h:h + 1], ref_r) <= 2e-4
+    assert max_abs(o[b:b + 1, h:h + 1], ref_r) <= 2e-2 and mean_rel(o[b:b + 1, h:h + 1], ref_r) <= 1e-2
+    for bb, hh in ((0, 0), (3, 31)):
+        sl = lambda t: t[bb:bb + 1, hh:hh + 1].contiguous()
+        assert torch.equal(M.attention_full_int8(sl(q8), sl(k8), sl(v8), sl(qs), sl(ks), sl(vs), False, sm), o_ref[bb:bb + 1, hh:hh + 1])
+
+
+@pytest.mark.parametrize("variant,B,H,H_kv,N,D,causal", [
+    ("full", 1, 12, 12, 4096, 128, False),     # 12 heads: 8 dealt whole to the XCDs, the workgroups of 4 cut into 8 runs
+    ("full", 3, 3, 3, 512, 64, True),          # 9 heads of 4 workgroups: the ninth is dealt one workgroup at a time
+    ("full", 1, 20, 10, 256, 128, True),       # 10 K/V heads shared by 20 query heads
+    ("full", 5, 1, 1, 300, 256, False),        # fewer heads than XCDs
+    ("half", 1, 12, 12, 1024, 128, True),
+    ("fp", 3, 5, 5, 640, 64, False),
+])
+def test_head_counts_that_do_not_divide_among_the_xcds(variant, B, H, H_kv, N, D, causal):
+    """Whatever the workgroup -> (batch, head, query block) mapping of a launch, every output slice must be computed exactly
+    once: the whole call reproduces, bit for bit, the calls on single (batch, K/V head) slices; one slice is also held
+    against the oracle."""
+    gen = torch.Generator(device=DEV).manual_seed(61)
+    mk = lambda h: torch.randn((B, h, N, D), generator=gen, device=DEV, dtype=torch.float16)
+    q, k, v = mk(H), mk(H_kv), mk(H_kv)
+    sm, grp = D ** -0.5, H // H_kv
+    if variant == "fp":
+        args = (q, k, v)
+        fn = lambda a: M.attention(*a, causal, sm)
+    else:
+        q8, qs = M.quant_pertoken(q)
+        k8, ks = M.quant_pertoken(k)
+        if variant == "half":
+            args = (q8, k8, v, qs, ks)
+            fn = lambda a: M.attention_int8(*a, causal, sm)
+        else:
+            v8, vs = M.quant_pertensor(v)
+            args = (q8, k8, v8, qs, ks, vs)
+            fn = lambda a: M.attention_full_int8(*a, causal, sm)
+    o = fn(args)
+    assert o.shape == (B, H, N, D) and torch.isfinite(o).all()
+    for b in range(B):
+        for hk in range(H_kv):
+            sl = lambda i, t: (t[b:b + 1, hk * grp:(hk + 1) * grp] if i in ((0,) if variant == "fp" else (0, 3))
+                               else t[b:b + 1, hk:hk + 1]).contiguous()
+            o1 = fn(tuple(sl(i, t) for i, t in enumerate(args)))
+            assert torch.equal(o1, o[b:b + 1, hk * grp:(hk + 1) * grp]), (b, hk)
+    b, hk = B - 1, H_kv - 1
+    h = hk * grp + grp - 1
+    cq = lambda t: t[b:b + 1, h:h + 1].cpu()
+    ck = lambda t: t[b:b + 1, hk:hk + 1].cpu()
+    bn = M.block_n(variant, D)
+    if variant == "fp":
+        ref = O.attention_fp(cq(q), ck(k), ck(v), causal, sm, block_n=bn)
+    elif variant == "half":
+        ref = O.attention_int8(cq(q8), ck(k8), ck(v), cq(qs), ck(ks), causal, sm, block_n=bn)
+    else:
+        ref = O.attention_full_int8(cq(q8), ck(k8), ck(v8), cq(qs), ck(ks), ck(vs), causal, sm, block_n=bn)
+    assert max_abs(o[b:b + 1, h:h + 1], ref) <= 4e-3 and mean_rel(o[b:b + 1, h:h + 1], ref) <= (2e-4 if variant == "full" else 6e-4)
 
 
 def test_constant_v_gives_constant_columns_at_full_size():
