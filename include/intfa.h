@@ -59,7 +59,7 @@ enum {
     INTFA_ERR_SHAPE = -7,         /* batch/heads not positive, a row stride below head_dim, a (batch, head) slice of
                                      k or v spanning 4 GiB or more, or sizes that overflow 32-bit block indices */
     INTFA_ERR_SPLITS = -8,        /* num_splits out of range */
-    INTFA_ERR_VSCALE = -9,        /* v_scale_block neither a multiple of the key-block length nor 64 at head_dim <= 128, or
+    INTFA_ERR_VSCALE = -9,        /* v_scale_block neither a multiple of the key-block length nor 64 at head_dim 128, or
                                      vs_stride_blk below head_dim */
     INTFA_ERR_SCRATCH = -10       /* intfa_fwd_full_int8_static: the call's split-KV partials exceed
                                      INTFA_STATIC_SCRATCH_BYTES, or the device index is beyond the table of 64 devices */
@@ -110,8 +110,8 @@ typedef struct intfa_fwd_params {
                                  causal the general kernels deal, per query block of 128 rows, the blocks VISIBLE to that
                                  query block (ceil(visible / num_splits) each, so no split of a query block is empty);
                                  decode-shaped calls (seqlen <= 64; every variant and head_dim, except full-int8 at
-                                 head_dim 256 with blocked V scales, which runs the general kernel) keep the partition of
-                                 the whole key sequence also with causal: split s takes blocks s * ceil(blocks /
+                                 head_dim 128 with v_scale_block = 64, which runs the general kernel) keep the partition
+                                 of the whole key sequence also with causal: split s takes blocks s * ceil(blocks /
                                  num_splits) onward, cut at the last visible block.  The requantisation frame of P depends
                                  on the ranges, so a bit-faithful CPU evaluation must use the same ones. */
     void*   workspace;        /* device scratch of at least intfa_fwd_workspace_bytes() bytes, or NULL */
@@ -130,11 +130,12 @@ typedef struct intfa_fwd_params {
                                  head_dim fp32 scales per block of keys (channel stride 1, row stride vs_stride_blk, batch
                                  and head strides vs_stride_b / vs_stride_h over heads_kv heads; 4-byte aligned, fp32 as in
                                  that kernel whatever scale_dtype says).  Must be a multiple of
-                                 intfa_fwd_block_n(INTFA_VARIANT_FULL_INT8, head_dim), or 64 at head_dim <= 128: the
-                                 granularity of the reference's kernel itself (kBlockN = 64 at head_dim 128,
-                                 csrc/flash_fwd_launch_template.h:514-519).  The softmax then still advances per 128-key
-                                 block (running maximum and P8 as intfa_fwd_block_n() says); P V is summed in int32 per
-                                 64-key half and each half is multiplied by its own scale row. */
+                                 intfa_fwd_block_n(INTFA_VARIANT_FULL_INT8, head_dim) (64, except 128 at head_dim 128),
+                                 or 64 at head_dim 128: the granularity of the reference's kernel itself (kBlockN = 64 at
+                                 head_dim 128, csrc/flash_fwd_launch_template.h:514-519).  At head_dim 128 the softmax
+                                 then still advances per 128-key block (running maximum and P8 as intfa_fwd_block_n()
+                                 says); P V is summed in int32 per 64-key half and each half is multiplied by its own
+                                 scale row. */
     int32_t reserved0;        /* set to 0 */
     int64_t vs_stride_blk;    /* elements between consecutive scale rows of v_scale (>= head_dim) */
     const int32_t* seqlens_k; /* optional device array [batch]: number of keys of each batch entry, 0 <= n <= seqlen_k (a
@@ -147,9 +148,9 @@ typedef struct intfa_fwd_params {
     int32_t causal_rows;      /* 0, or the number of query positions when the row axis holds several query heads of one
                                  K/V group one after the other (decoding with grouped heads described as heads = heads_kv,
                                  seqlen = group * positions, see heads_kv): row r is position r % causal_rows for the causal
-                                 mask.  Only with causal and the shapes of the decode kernels: seqlen <= 64 and
-                                 head_dim <= 128 (not with v_scale_block = 64) or head_dim 256 (not with blocked V
-                                 scales), any variant.  seqlen must be a multiple of it. */
+                                 mask.  Only with causal and the shapes of the decode kernels: seqlen <= 64, any variant
+                                 and head_dim (not with v_scale_block = 64 at head_dim 128).  seqlen must be a multiple
+                                 of it. */
     int32_t reserved1;        /* set to 0 */
 } intfa_fwd_params;
 
@@ -161,8 +162,10 @@ const char* intfa_error_string(int code);
 
 /* Key-block length of a variant at a head_dim (the reference's BLOCK_N, an autotuned value there:
  * configs.py:13-19).  The running max and, on the full-int8 path, the requantisation of P advance per key block,
- * so a bit-faithful CPU evaluation must use the same value.  It holds for every shape: the kernel that takes over
- * decode-shaped calls (at most 64 query rows, head_dim <= 128) walks the same blocks.
+ * so a bit-faithful CPU evaluation must use the same value.  Full-int8: 128 at head_dim 128, 64 otherwise; half-int8 and
+ * fp16: 64.  At head_dim >= 64 that is a length the reference's kernel admits (flash_atten_full_int8.py:88,
+ * static_assert BLOCK_N <= HEAD_DIM); head_dim 16 and 32 are computed zero-padded to 64 and keep the 64-key block.  It holds for every shape: the kernel
+ * that takes over decode-shaped calls (at most 64 query rows) walks the same blocks.
  * Negative INTFA_ERR_* for unknown arguments. */
 int intfa_fwd_block_n(int variant, int head_dim);
 

@@ -79,6 +79,43 @@ def test_static_scratch_entry_point_equals_the_workspace_entry_point_on_two_call
     assert torch.equal(o_st, o_ws) and torch.equal(lse_st, lse_ws)
 
 
+def test_static_scratch_entry_point_records_into_a_graph():
+    """After its first call on a device the entry point allocates, frees and synchronises nothing: a stream capture, which
+    any of those would break, records it (forward and combine kernels), and replays on inputs changed in between give the
+    bits of the workspace entry point."""
+    lib = _capi.load()
+    pb = make_problem(2, 4, 200, 1024, 128, seed=904, causal=True)
+    splits = 3
+    shape = (pb["B"], pb["H"], pb["Nq"], pb["D"])
+    out = torch.full(shape, float("nan"), dtype=torch.float16, device=DEV)
+    lse = torch.full(shape[:3], float("nan"), dtype=torch.float32, device=DEV)
+    p = fill(pb, out, lse, splits)
+    p.workspace, p.workspace_bytes = None, 0
+
+    def call_static():
+        rc = lib.intfa_fwd_full_int8_static(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, lib.intfa_error_string(rc)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                 # the first call on the device looks up the scratch array: outside the capture
+        call_static()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call_static()
+    g = torch.Generator(device=DEV).manual_seed(905)
+    for rep in range(3):
+        q = torch.randn(shape, generator=g, device=DEV, dtype=torch.float16)
+        pb["t"][0].copy_((q * 40).round().clamp(-127, 127).to(torch.int8))      # new int8 Q, written by eager kernels
+        out.fill_(float("nan")); lse.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        (o_ws, lse_ws), _ = run_both(pb, splits)
+        assert torch.equal(out, o_ws) and torch.equal(lse, lse_ws), rep
+
+
 def test_static_scratch_entry_point_rejects_what_does_not_fit():
     lib = _capi.load()
     pb = make_problem(1, 1, 8, 256, 128, seed=903, causal=False)
