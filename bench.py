@@ -106,7 +106,7 @@ WORKLOADS = {
 # them, NOT measured in the run that prints them (counters need the profiler); workloads without a profile report None.
 MEASURED_TRAFFIC_BYTES = {
     # FETCH_SIZE x 1.9997 + WRITE_SIZE x 1.0 (KiB per dispatch, factors from a 256 MiB copy): 194.3 MiB read + 128 MiB written
-    "full_int8_B4_H32_N4096_d128": (337909687, "profiles/fwd_full_int8_d128_B4_H32_N4096.txt"),
+    "full_int8_B4_H32_N4096_d128": (337941934, "profiles/fwd_full_int8_d128_B4_H32_N4096.txt"),
     # FETCH_SIZE x 1.9998 + WRITE_SIZE 256 x 1.0: 1032.2 MiB read + 0.25 MiB written (algorithmic: 1082523648)
     "full_int8_decode_B32_H32_Nq1_Nk4096_d128": (1082595402, "profiles/fwd_decode_full_int8_d128_B32_H32_Nq1_Nk4096.txt"),
 }
@@ -397,6 +397,11 @@ def main():
                            "traffic": traffic_of(args.workload)[0], "traffic_source": traffic_of(args.workload)[1],
                            "kernel": "fwd_decode_full_int8_kernel" if variant == "full" else "fwd_decode_f16pv_kernel", "avg_launch_ms": kern_ms, "median_launch_ms": kern_med_ms,
                            "launch_includes": "forward kernel" + (" + split-KV combine kernel" if splits != 1 else "")}
+        if other_round is not None:         # the same bytes over the other rounding's launch time
+            g_o = alg_bytes / (other_round["avg_launch_ms"] * 1e-3) / 1e9
+            out["roofline_" + other_round["p_round"] + "_rounding"].update(
+                {"bound": "hbm", "achieved": g_o, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g_o / HBM_PEAK_GBS,
+                 "kernel": out["roofline"]["kernel"]})
     if parity is not None:
         out["parity"] = parity
     if args.cpu_seconds > 0:
