@@ -39,6 +39,20 @@ def build_c_caller(verbose: bool = True) -> str:
     return C_CALLER
 
 
+RATE_PROBE_SRC = os.path.join(os.path.dirname(HERE), "bench_rate_probe.hip")
+RATE_PROBE = RATE_PROBE_SRC[:-4]
+
+
+def build_rate_probe(verbose: bool = True) -> str:
+    """Compiles the stand-alone instruction-rate probe beside bench.py (measurement only; no library code in it)."""
+    r = subprocess.run(["hipcc", *[f for f in FLAGS if f != "-fPIC"], RATE_PROBE_SRC, "-o", RATE_PROBE], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {RATE_PROBE_SRC}:\n{r.stderr[-4000:]}")
+    if verbose:
+        print(f"built {RATE_PROBE}")
+    return RATE_PROBE
+
+
 def build(verbose: bool = True, jobs: int = 8, only=None) -> str:
     """Compiles every source and links the library.  `only` (development): a list of name fragments - sources whose file
     name contains none of them keep their existing object file."""
@@ -84,6 +98,8 @@ def build(verbose: bool = True, jobs: int = 8, only=None) -> str:
         print(f"built {OUT} from {len(srcs)} source file(s), {len(todo)} compiled")
     if os.path.exists(C_CALLER_SRC):
         build_c_caller(verbose)
+    if os.path.exists(RATE_PROBE_SRC) and not only:
+        build_rate_probe(verbose)
     return OUT
 
 
