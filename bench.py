@@ -77,6 +77,8 @@ WORKLOADS = {
     "full_int8_B4_H32_N16384_d64": dict(variant="full", B=4, H=32, N=16384, D=64, causal=False, splits=1),
     "half_int8_B4_H32_N4096_d64": dict(variant="half", B=4, H=32, N=4096, D=64, causal=False, splits=1),
     "fp16_B4_H32_N4096_d64": dict(variant="fp", B=4, H=32, N=4096, D=64, causal=False, splits=1),
+    "fp16_B4_H32_N4096_d64_causal": dict(variant="fp", B=4, H=32, N=4096, D=64, causal=True, splits=1),
+    "half_int8_B4_H32_N4096_d64_causal": dict(variant="half", B=4, H=32, N=4096, D=64, causal=True, splits=1),
     # a number of (batch, head) pairs that is no multiple of the eight XCDs (how whole heads are pinned to one L2 then)
     "full_int8_B1_H12_N4096_d128": dict(variant="full", B=1, H=12, N=4096, D=128, causal=False, splits=1),
     # head_dim 256 at the headline's batch, heads and length (the eight-wave kernel of that head_dim)

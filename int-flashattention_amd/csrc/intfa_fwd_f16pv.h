@@ -43,7 +43,9 @@ template <int D> struct F16PvGeom {
 // (16-bit K tiles at head_dim 256 are 32 KiB each: double-buffered beside the V tiles they leave room for one workgroup
 // per compute unit, whatever the register count)
 template <bool QK_INT8, int D, bool CAUSAL, int IO_DT, bool SPLIT>
-__global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f16pv_kernel(const KParams p) {
+// (head_dim 64: three waves per SIMD - the non-causal instances need 140-146 registers, the masked ones are held to 168
+// and spill 7-9; 33 KiB / 25 KiB of LDS allow it)
+__global__ void __launch_bounds__(kThreads, D > 128 ? (QK_INT8 ? 2 : 1) : (D == 64 ? 3 : 2)) fwd_f16pv_kernel(const KParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr int BN = kBlockN16, NST = BN / 32;
     constexpr int QB = QK_INT8 ? 1 : 2;               // bytes per Q/K element
@@ -246,7 +248,7 @@ __global__ void __launch_bounds__(kThreads, (QK_INT8 || D <= 128) ? 2 : 1) fwd_f
         // sum p' v and for the row sum, so acc / l and m + log2(l) are unchanged; only the 16-bit rounding of the single
         // p' lands on other values (relative 2^-12, unbiased).  In the common case no vector instruction touches the output.
         const float mxs = mx * qsc;
-        if (__builtin_expect(__builtin_amdgcn_ballot_w64(mxs > m_run + kFrameSlack) != 0, 0)) {
+        if (DIAG || __builtin_expect(__builtin_amdgcn_ballot_w64(mxs > m_run + kFrameSlack) != 0, 0)) {   // (the few masked blocks always move the frame: no branch around the rescale there)
             const float m_mv = fmaxf(m_run, mxs);
             const float a_mv = fast_exp2(m_run - m_mv);
             m_run = m_mv;
