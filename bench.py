@@ -108,7 +108,7 @@ WORKLOADS = {
 # them, NOT measured in the run that prints them (counters need the profiler); workloads without a profile report None.
 MEASURED_TRAFFIC_BYTES = {
     # FETCH_SIZE x 1.9997 + WRITE_SIZE x 1.0 (KiB per dispatch, factors from a 256 MiB copy): 194.3 MiB read + 128 MiB written
-    "full_int8_B4_H32_N4096_d128": (337942449, "profiles/fwd_full_int8_d128_B4_H32_N4096.txt"),
+    "full_int8_B4_H32_N4096_d128": (337941156, "profiles/fwd_full_int8_d128_B4_H32_N4096.txt"),
     # FETCH_SIZE x 1.9998 + WRITE_SIZE 256 x 1.0: 1032.2 MiB read + 0.25 MiB written (algorithmic: 1082523648)
     "full_int8_decode_B32_H32_Nq1_Nk4096_d128": (1082595402, "profiles/fwd_decode_full_int8_d128_B32_H32_Nq1_Nk4096.txt"),
 }
